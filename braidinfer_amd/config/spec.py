@@ -94,6 +94,9 @@ class ScheduleEntry:
     writes_cache: bool = True
     # cache units of the layer's further mixers, by their role in `LayerSpec.more_mixers`
     more_caches: Dict[str, int] = field(default_factory=dict)
+    # the embedding output (the rows as they were before the first entry ran) is added to the residual rows
+    # right before this entry runs: a stack that passes some layers several times feeds the input in again
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -115,6 +118,8 @@ class ModelSpec:
     lm_head_prefix: str
     stop_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
+    # tensor-name prefix of a position encoding's tensors, by the encoding's name (absent: "position.<name>.")
+    position_prefixes: Dict[str, str] = field(default_factory=dict)
 
 
 def default_schedule(n_layers: int) -> List[ScheduleEntry]:

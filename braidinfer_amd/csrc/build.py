@@ -38,6 +38,7 @@ MODULES: Dict[str, List[str]] = {
     "random_weights": ["random_weights.hip"],
     "pooled_attention": ["pooled_attention.hip"],
     "gated_recurrence": ["gated_recurrence.hip"],
+    "delta_rule": ["delta_rule.hip"],
     "latent_attention": ["latent_attention.hip"],
     "routed_experts": ["routed_experts.hip"],
 }

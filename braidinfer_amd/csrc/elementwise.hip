@@ -541,6 +541,27 @@ extern "C" int br_residual_add(float* x, const void* y, int y_is_bf16, size_t n,
     return br_check_launch();
 }
 
+// ------------------------------------------------------- learnt position rows ------
+// x[t, :] += float(table[pos[t], :]): a learnt vector per position joins the embedding.  grid (T).
+template <typename T>
+__global__ void add_position_rows_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ pos,
+                                         int H, int n_rows) {
+    const int p = pos[blockIdx.x];
+    if (p < 0 || p >= n_rows) return;
+    const T* row = table + (size_t)p * H;
+    float* xr = x + (size_t)blockIdx.x * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) xr[i] += to_f32<T>(row[i]);
+}
+
+extern "C" int br_add_position_rows(float* x, const void* table, int is_bf16, const int* pos, int T, int H, int n_rows,
+                                    hipStream_t s) {
+    if (T <= 0 || H <= 0) return BR_OK;
+    if (n_rows <= 0) return BR_BAD_ARG;
+    if (is_bf16) add_position_rows_kernel<bf16><<<T, 256, 0, s>>>(x, (const bf16*)table, pos, H, n_rows);
+    else add_position_rows_kernel<float><<<T, 256, 0, s>>>(x, (const float*)table, pos, H, n_rows);
+    return br_check_launch();
+}
+
 // ------------------------------------------------------------------ row gather -----
 // out[i, :] = x[rows[i], :] (float)   reference: D2dCopy of the last row,
 // megakernel/megakernel_compile.rs:522-527.

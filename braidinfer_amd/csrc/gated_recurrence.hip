@@ -630,11 +630,13 @@ extern "C" int br_shift_mix(const void* h, int is_bf16, const float* mu, void* o
 // ------------------------------------------------ head norm, weight and gate --------
 // y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w[h, :] * silu(gate[t, h, :]): every head's output
 // divided by its root mean square, a weight per head and channel, and a gate from the float sums of its
-// projection (rows `gate_stride` floats apart).  16 lanes a (token, head) row as in `glr_head_norm_kernel`.
+// projection (rows `gate_stride` floats apart; `gate_sigmoid`: sigmoid of the sums instead of silu).  16 lanes a
+// (token, head) row as in `glr_head_norm_kernel`.
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                              const float* __restrict__ gate, size_t gate_stride,
-                                                             T* __restrict__ y, size_t n_rows, int H, int e, float eps) {
+                                                             T* __restrict__ y, size_t n_rows, int H, int e, float eps,
+                                                             int gate_sigmoid) {
     const size_t r = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
     const int l = threadIdx.x & 15;
     const bool on = r < n_rows;
@@ -651,19 +653,19 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
     for (int i = l; i < e; i += 16) {
         float v = orow[i] * inv;
         if (wrow) v *= wrow[i];
-        if (grow) { const float z = grow[i]; v *= z / (1.0f + expf(-z)); }
+        if (grow) { const float z = grow[i]; v *= (gate_sigmoid ? 1.0f : z) / (1.0f + expf(-z)); }
         yrow[i] = from_f32<T>(v);
     }
 }
 
 extern "C" int br_head_norm_gate(const float* o, const float* w, const float* gate, size_t gate_stride, void* y, int y_is_bf16,
-                                 int T, int H, int e, float eps, hipStream_t s) {
+                                 int T, int H, int e, float eps, int gate_sigmoid, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (H <= 0 || e <= 0 || (gate && gate_stride < (size_t)H * e)) return BR_BAD_ARG;
     const size_t n_rows = (size_t)T * H;
     const unsigned blocks = (unsigned)((n_rows + 15) / 16);
-    if (y_is_bf16) head_norm_gate_kernel<bf16><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (bf16*)y, n_rows, H, e, eps);
-    else head_norm_gate_kernel<float><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (float*)y, n_rows, H, e, eps);
+    if (y_is_bf16) head_norm_gate_kernel<bf16><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (bf16*)y, n_rows, H, e, eps, gate_sigmoid);
+    else head_norm_gate_kernel<float><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (float*)y, n_rows, H, e, eps, gate_sigmoid);
     return br_check_launch();
 }
 

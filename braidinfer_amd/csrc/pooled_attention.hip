@@ -23,7 +23,10 @@
 #define MAX_EPL 8   // head widths up to 64 * MAX_EPL
 
 // ------------------------------------------------------------------- prepare -------
-// qkv [T, nq*dk + nkv*dk + nkv*dv] float (the product's float sums), one wave per (token, head).
+// qkv [T, width] float (the product's float sums: queries, keys, and the values from column `v_col0` on, which is
+// nq*dk + nkv*dk when they have a projection of their own and nq*dk when the keys' sums, before their norm, are the
+// values too), one wave per (token, head).  `q_every` > 0: the query is multiplied by
+// 1 + q_coef ln(floor((p + 1) / q_every) + 1) at position p, behind its norm.
 // vf_role: 0 none, 1 this layer's values are written to `v_first`, 2 values become
 // (1 - lambda) v + lambda v_first.  Tokens of padding sequences (slot < 0) store nothing.
 template <typename T>
@@ -34,14 +37,13 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     const int* __restrict__ slots, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ q_out, T* __restrict__ storage, float* __restrict__ v_first,
     const float* __restrict__ lambda, int vf_role, int nq, int nkv, int dk, int dv, int page,
-    int write_cache) {
+    int write_cache, int width, int v_col0, float q_coef, int q_every) {
     extern __shared__ float row[];          // [max(dk, dv)]
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int width = nq * dk + nkv * dk + nkv * dv;
     const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
     const int kvh = is_q ? 0 : (is_k ? h - nq : h - nq - nkv);
     const int n = (is_q || is_k) ? dk : dv;
-    const int col0 = is_q ? h * dk : (is_k ? nq * dk + kvh * dk : nq * dk + nkv * dk + kvh * dv);
+    const int col0 = is_q ? h * dk : (is_k ? nq * dk + kvh * dk : v_col0 + kvh * dv);
     const float* src = qkv + (size_t)t * width + col0;
     const int slot = slots[seq_of_token[t]];
     const int p = pos[t];
@@ -76,6 +78,11 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
                 const int i = lane + 64 * j;
                 if (i < n) v[j] = v[j] * inv * nw[i];
             }
+        }
+        if (is_q && q_every > 0) {          // the query's temperature: it grows with the logarithm of the position
+            const float temp = 1.0f + q_coef * logf((float)((p + 1) / q_every) + 1.0f);
+#pragma unroll
+            for (int j = 0; j < MAX_EPL; ++j) v[j] *= temp;
         }
     }
     if (rd > 0) {                           // the barrier is met whatever the head
@@ -130,12 +137,11 @@ __global__ __launch_bounds__(256) void pwa_values_kernel(
     const float* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ pos,
     const int* __restrict__ seq_of_token, const int* __restrict__ slots, const int* __restrict__ block_table,
     int table_stride, T* __restrict__ storage, float* __restrict__ v_first, const float* __restrict__ lambda,
-    int vf_role, int n_tokens, int nq, int nkv, int dk, int dv, int page) {
+    int vf_role, int n_tokens, int nq, int nkv, int dk, int dv, int page, int width, int v_col0) {
     __shared__ float tile[64][65];
     const int t0 = blockIdx.x * 64, kvh = blockIdx.y, c0 = blockIdx.z * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int width = nq * dk + nkv * dk + nkv * dv;
-    const int col0 = nq * dk + nkv * dk + kvh * dv;
+    const int col0 = v_col0 + kvh * dv;
     const float lam = vf_role == 2 ? lambda[0] : 0.f;
     const int ch = c0 + lane;
     for (int r = 0; r < 16; ++r) {
@@ -170,8 +176,11 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
                               const float* cs, const float* sn, int rd, const int* pos, const int* seq_of_token,
                               const int* slots, const int* block_table, int table_stride, void* q_out,
                               void* storage, int is_bf16, float* v_first, const float* lambda, int vf_role,
-                              int T, int nq, int nkv, int dk, int dv, int page, int write_cache, hipStream_t s) {
+                              int T, int nq, int nkv, int dk, int dv, int page, int write_cache, int width, int v_from_k,
+                              float q_coef, int q_every, hipStream_t s) {
     if (T <= 0) return BR_OK;
+    const int v_col0 = v_from_k ? nq * dk : nq * dk + nkv * dk;
+    if (width < v_col0 + nkv * dv || (v_from_k && dv != dk) || (bias && v_from_k) || q_every < 0) return BR_BAD_ARG;
     if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL ||
         rd < 0 || rd > dk || (rd & 1) || page <= 0 || nq + 2 * nkv > 65535 || (rd > 0 && (!cs || !sn)) ||
         (vf_role && !v_first) || (vf_role == 2 && !lambda) || vf_role < 0 || vf_role > 2)
@@ -183,20 +192,45 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
     if (is_bf16)
         pwa_prepare_kernel<bf16><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                        block_table, table_stride, (bf16*)q_out, (bf16*)storage, v_first,
-                                                       lambda, vf_role, nq, nkv, dk, dv, page, write_cache);
+                                                       lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every);
     else
         pwa_prepare_kernel<float><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                         block_table, table_stride, (float*)q_out, (float*)storage,
-                                                        v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache);
+                                                        v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every);
     int rc = br_check_launch();
     if (rc != BR_OK || !tiled) return rc;
     dim3 vgrid((T + 63) / 64, nkv, (dv + 63) / 64);
     if (is_bf16)
         pwa_values_kernel<bf16><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (bf16*)storage,
-                                                      v_first, lambda, vf_role, T, nq, nkv, dk, dv, page);
+                                                      v_first, lambda, vf_role, T, nq, nkv, dk, dv, page, width, v_col0);
     else
         pwa_values_kernel<float><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (float*)storage,
-                                                       v_first, lambda, vf_role, T, nq, nkv, dk, dv, page);
+                                                       v_first, lambda, vf_role, T, nq, nkv, dk, dv, page, width, v_col0);
+    return br_check_launch();
+}
+
+// ----------------------------------------------------------------- output gate -----
+// o[t, h, i] <- o[t, h, i] * sigmoid(gate) * scale, with one gate number per element (gate row [nq * dv]) or one per
+// head (gate row [nq]); the gate's rows are float sums `gate_stride` apart.  grid (T), 256 threads.
+template <typename T>
+__global__ __launch_bounds__(256) void pwa_gate_kernel(T* __restrict__ o, const float* __restrict__ gate, size_t gate_stride,
+                                                       int nq, int dv, int per_head, float scale) {
+    const size_t t = blockIdx.x;
+    const int n = nq * dv;
+    const float* grow = gate + t * gate_stride;
+    T* orow = o + t * n;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const float z = grow[per_head ? i / dv : i];
+        orow[i] = from_f32<T>(to_f32<T>(orow[i]) * (scale / (1.0f + expf(-z))));
+    }
+}
+
+extern "C" int br_pwa_gate(void* o, int is_bf16, const float* gate, size_t gate_stride, int T, int nq, int dv, int per_head,
+                           float scale, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (nq <= 0 || dv <= 0 || gate_stride < (size_t)(per_head ? nq : nq * dv)) return BR_BAD_ARG;
+    if (is_bf16) pwa_gate_kernel<bf16><<<T, 256, 0, s>>>((bf16*)o, gate, gate_stride, nq, dv, per_head, scale);
+    else pwa_gate_kernel<float><<<T, 256, 0, s>>>((float*)o, gate, gate_stride, nq, dv, per_head, scale);
     return br_check_launch();
 }
 

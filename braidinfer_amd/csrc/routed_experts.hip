@@ -17,7 +17,7 @@
 
 // grid (T), one wave a token.
 __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ scores, const float* __restrict__ bias,
-                                                        int* __restrict__ chosen, float* __restrict__ share, int E, int top) {
+                                                        int* __restrict__ chosen, float* __restrict__ share, int E, int top, float out_scale) {
     const int t = blockIdx.x, lane = threadIdx.x;
     float z[RX_MAX_PER_LANE];
 #pragma unroll
@@ -50,14 +50,14 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
         for (int i = 0; i < RX_MAX_PER_LANE; ++i)
             if (lane + 64 * i == at) z[i] = -INFINITY;
     }
-    if (lane < top) share[(size_t)t * top + lane] = mine / total;
+    if (lane < top) share[(size_t)t * top + lane] = mine / total * out_scale;
 }
 
 extern "C" int br_route_topk(const float* scores, const float* bias, int* chosen, float* share, int T, int E, int top,
-                             hipStream_t s) {
+                             float out_scale, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (E <= 0 || E > 64 * RX_MAX_PER_LANE || top <= 0 || top > E || top > 64) return BR_BAD_ARG;
-    route_topk_kernel<<<T, 64, 0, s>>>(scores, bias, chosen, share, E, top);
+    route_topk_kernel<<<T, 64, 0, s>>>(scores, bias, chosen, share, E, top, out_scale);
     return br_check_launch();
 }
 

@@ -140,7 +140,7 @@ class DecoderModel:
         yield self.final_norm, s.final_norm_prefix
         yield self.lm_head, s.lm_head_prefix
         for name, p in self.positions.items():
-            yield p, f"position.{name}."
+            yield p, s.position_prefixes.get(name, f"position.{name}.")
 
     def weight_specs(self) -> List[TensorSpec]:
         out: List[TensorSpec] = []
@@ -242,10 +242,18 @@ class DecoderModel:
             enc.add_to_embedding(x, step)
         if probe is not None:
             probe("embed", x)
+        x0 = None
+        if any(e.adds_embedding for e in self.schedule):
+            # entries that add the embedding output again read a copy: the rows themselves move on
+            x0 = ws.get("embedding_out", (T, H), torch.float32)
+            x0.copy_(x)
         step.prepared_norm = None
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             step.schedule_index = i
+            if e.adds_embedding:
+                K.residual_add(x, x0)
+                step.prepared_norm = None          # what a product prepared for the next norm is of the rows before the sum
             # the norm that reads the residual rows after this layer: the next scheduled layer's first
             # (the final norm reads chosen rows only and is left alone)
             step.norm_after_layer = None

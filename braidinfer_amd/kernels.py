@@ -193,6 +193,18 @@ def residual_add(x: torch.Tensor, y: torch.Tensor) -> None:
     _check(f(_ptr(x), _ptr(y), _is_bf16(y, "residual_add"), x.numel(), _stream()), "residual_add")
 
 
+def add_position_rows(x: torch.Tensor, table: torch.Tensor, positions: torch.Tensor) -> None:
+    """x[t, :] += table[positions[t], :]: x float [T, H], table [rows, H] float or bfloat16, positions int32 [T]
+    (a position outside the table adds nothing; callers refuse such steps on the host)."""
+    _dev("add_position_rows", x, table, positions)
+    T, H = x.shape
+    _req(x.dtype == torch.float32 and table.dim() == 2 and table.shape[1] == H, "add_position_rows: x float32 [T, H], table [rows, H]")
+    _req(positions.dtype == torch.int32 and positions.numel() >= T, "add_position_rows: positions int32 [T]")
+    f = _fn("elementwise", "br_add_position_rows", [_P, _P, c_int, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(x), _ptr(table), _is_bf16(table, "add_position_rows"), _ptr(positions), T, H, table.shape[0], _stream()),
+           "add_position_rows")
+
+
 def gather_rows(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
     _dev("gather_rows", x, rows, out)
     _req(x.dtype == torch.float32 and out.dtype == torch.float32 and rows.dtype == torch.int32, "gather_rows: dtypes")
@@ -528,16 +540,21 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
                 rotary_dim: int, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
                 block_table: torch.Tensor, q_out: torch.Tensor, unit: torch.Tensor, v_first: Optional[torch.Tensor],
                 mix: Optional[torch.Tensor], v_role: int, nq: int, nkv: int, dk: int, dv: int, page: int,
-                write_cache: bool) -> None:
-    """Float projection sums [T, nq*dk + nkv*dk + nkv*dv] -> queries (normed, rotated) in `q_out` and the
-    tokens' keys (normed, rotated) and values in their cache pages.  `v_role` 1 leaves the values in
-    `v_first`, 2 mixes them with it by the scalar `mix`."""
+                write_cache: bool, values_from_keys: bool = False, q_temp_coef: float = 0.0, q_temp_every: int = 0) -> None:
+    """Float projection sums [T, nq*dk + nkv*dk + nkv*dv (+ more columns that are not read)] -> queries (normed,
+    rotated) in `q_out` and the tokens' keys (normed, rotated) and values in their cache pages.  `v_role` 1 leaves
+    the values in `v_first`, 2 mixes them with it by the scalar `mix`.  `values_from_keys`: there are no value
+    columns, the keys' sums as projected (before norm and rotation) are the values.  `q_temp_every` > 0: the query
+    at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) behind its norm."""
     _dev("pwa_prepare", qkv, bias, q_norm, k_norm, cos, sin, positions, seq_of_token, slots, block_table, q_out, unit,
          v_first, mix)
     T = qkv.shape[0]
-    width = nq * dk + nkv * dk + nkv * dv
-    _req(qkv.dtype == torch.float32 and qkv.shape == (T, width), "pwa_prepare: projections must be float32 [T, nq*dk + nkv*(dk+dv)]")
+    width = nq * dk + nkv * dk + (0 if values_from_keys else nkv * dv)
+    _req(qkv.dtype == torch.float32 and qkv.dim() == 2 and qkv.shape[1] >= width,
+         "pwa_prepare: projections must be float32 [T, nq*dk + nkv*(dk+dv) or more]")
+    _req(not values_from_keys or (dv == dk and bias is None), "pwa_prepare: values taken from the keys have their width and no bias")
     _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "pwa_prepare: bias float32 of the projections' width")
+    _req(q_temp_every >= 0, "pwa_prepare: the query temperature's period must not be negative")
     for nw in (q_norm, k_norm):
         _req(nw is None or (nw.dtype == torch.float32 and nw.numel() == dk), "pwa_prepare: norm weights float32 [dk]")
     _req(positions.numel() >= T and seq_of_token.numel() >= T, "pwa_prepare: positions shorter than tokens")
@@ -552,11 +569,26 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
              "pwa_prepare: v_first float32 [T, nkv*dv]")
         _req(v_role != 2 or (mix is not None and mix.dtype == torch.float32 and mix.numel() == 1), "pwa_prepare: mix is one float")
     f = _fn("pooled_attention", "br_pwa_prepare",
-            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 8 + [_P])
+            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 10 + [c_float, c_int, _P])
     _check(f(_ptr(qkv), _ptr(bias), _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(cos), _ptr(sin), int(rotary_dim),
              _ptr(positions), _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(q_out),
              _ptr(unit), _is_bf16(unit, "pwa_prepare"), _ptr(v_first), _ptr(mix), int(v_role), T, nq, nkv, dk, dv, page,
-             int(write_cache), _stream()), "pwa_prepare")
+             int(write_cache), int(qkv.shape[1]), int(bool(values_from_keys)), float(q_temp_coef), int(q_temp_every),
+             _stream()), "pwa_prepare")
+
+
+def pwa_gate(o: torch.Tensor, gate: torch.Tensor, nq: int, dv: int, per_head: bool, scale: float = 1.0) -> None:
+    """o[t, h, i] <- o[t, h, i] * sigmoid(g) * scale in place, g = gate[t, h] (`per_head`) or gate[t, h * dv + i]:
+    o [T, nq*dv]; gate a float view [T, nq or nq*dv] whose rows may be strided (the sums of its projection)."""
+    _dev("pwa_gate", o)
+    T = o.shape[0]
+    n = nq if per_head else nq * dv
+    _req(o.shape == (T, nq * dv), "pwa_gate: o [T, nq*dv]")
+    _req(gate.is_cuda and gate.dtype == torch.float32 and gate.shape == (T, n) and gate.stride(1) == 1,
+         "pwa_gate: gate float32 [T, heads] or [T, heads * value width]")
+    gs = gate.stride(0) if T > 1 else n
+    f = _fn("pooled_attention", "br_pwa_gate", [_P, c_int, _P, c_size_t, c_int, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(o), _is_bf16(o, "pwa_gate"), _ptr(gate), gs, T, nq, dv, int(bool(per_head)), float(scale), _stream()), "pwa_gate")
 
 
 def pwa_pool(unit: torch.Tensor, block_table: torch.Tensor, pooled: torch.Tensor, pooled_table: torch.Tensor,
@@ -810,9 +842,9 @@ def shift_mix(h: torch.Tensor, mu: torch.Tensor, out: torch.Tensor, kept: torch.
 
 
 def head_norm_gate(o: torch.Tensor, w: Optional[torch.Tensor], gate: Optional[torch.Tensor], out: torch.Tensor, H: int, e: int,
-                   eps: float) -> None:
-    """out[t, h, :] = o[t, h, :] / rms * w[h, :] * silu(gate[t, h, :]): o float [T, H*e], w float [H*e] or None, gate a float
-    view [T, H*e] whose rows may be strided (the sums of its projection) or None."""
+                   eps: float, gate_sigmoid: bool = False) -> None:
+    """out[t, h, :] = o[t, h, :] / rms * w[h, :] * silu(gate[t, h, :]) (`gate_sigmoid`: sigmoid instead of silu): o float
+    [T, H*e], w float [H*e] or None, gate a float view [T, H*e] whose rows may be strided (the sums of its projection) or None."""
     _dev("head_norm_gate", o, w, out)
     T = o.shape[0]
     _req(o.dtype == torch.float32 and o.shape == (T, H * e) and out.shape == (T, H * e), "head_norm_gate: o float32 [T, H*e]")
@@ -821,8 +853,68 @@ def head_norm_gate(o: torch.Tensor, w: Optional[torch.Tensor], gate: Optional[to
     if gate is not None:
         _req(gate.is_cuda and gate.dtype == torch.float32 and gate.shape == (T, H * e) and gate.stride(1) == 1, "head_norm_gate: gate float32 [T, H*e]")
         gs = gate.stride(0) if T > 1 else H * e
-    f = _fn("gated_recurrence", "br_head_norm_gate", [_P, _P, _P, c_size_t, _P, c_int, c_int, c_int, c_int, c_float, _P])
-    _check(f(_ptr(o), _ptr(w), _ptr(gate), gs, _ptr(out), _is_bf16(out, "head_norm_gate"), T, H, e, float(eps), _stream()), "head_norm_gate")
+    f = _fn("gated_recurrence", "br_head_norm_gate", [_P, _P, _P, c_size_t, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P])
+    _check(f(_ptr(o), _ptr(w), _ptr(gate), gs, _ptr(out), _is_bf16(out, "head_norm_gate"), T, H, e, float(eps),
+             int(bool(gate_sigmoid)), _stream()), "head_norm_gate")
+
+
+# ------------------------------------------------- recurrences with one decay a head -----
+def dr_conv_prepare(rows: torch.Tensor, taps: torch.Tensor, kept: Optional[torch.Tensor], a_log: torch.Tensor,
+                    dt_bias: torch.Tensor, seq_of_token: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor,
+                    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: torch.Tensor, B: int, G: int, H: int, d: int,
+                    e: int) -> None:
+    """rows float [T, >= C + 2 H] with C = 2 G d + H e: the sums q | k | v | b | a of a gated delta rule's projections.
+    The first C columns pass a causal convolution over time per channel (taps float [C, n], the last column the current
+    token's; `kept` a float view [slots, (n - 1) * C] of every sequence's last inputs, read and then brought up to
+    date) and silu; q and k become unit vectors per head (q times d^-1/2); gb [T, 2 H] takes
+    g = exp(-exp(a_log) softplus(a + dt_bias)) and beta = sigmoid(b)."""
+    _dev("dr_conv_prepare", rows, taps, a_log, dt_bias, seq_of_token, cu_seqlens, slots, q, k, v, gb)
+    T = rows.shape[0]
+    C = 2 * G * d + H * e
+    n = taps.shape[1] if taps.dim() == 2 else 0
+    _req(rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape[1] >= C + 2 * H, "dr_conv_prepare: rows float32 [T, >= C + 2 H]")
+    _req(taps.dtype == torch.float32 and taps.shape == (C, n) and 1 <= n <= 16, "dr_conv_prepare: taps float32 [C, 1..16]")
+    _req(a_log.dtype == dt_bias.dtype == torch.float32 and a_log.numel() == H and dt_bias.numel() == H, "dr_conv_prepare: A_log and dt_bias float32 [H]")
+    _req(q.dtype == k.dtype == v.dtype == gb.dtype == torch.float32 and q.shape == k.shape == (T, G * d) and v.shape == (T, H * e)
+         and gb.shape == (T, 2 * H), "dr_conv_prepare: q, k [T, G d], v [T, H e], gb [T, 2 H] float32")
+    _req(seq_of_token.numel() >= T and cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "dr_conv_prepare: arrays shorter than the batch")
+    ks = 0
+    if n > 1:
+        _req(kept is not None and kept.is_cuda and kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] == (n - 1) * C
+             and kept.stride(1) == 1, "dr_conv_prepare: kept float32 [slots, (n - 1) * C]")
+        ks = kept.stride(0)
+    f = _fn("delta_rule", "br_dr_conv_prepare", [_P, c_int, _P, c_int, _P, c_size_t, _P, _P, _P, _P, _P, _P, _P, _P, _P] + [c_int] * 6 + [_P])
+    _check(f(_ptr(rows), int(rows.shape[1]), _ptr(taps), n, _ptr(kept) if n > 1 else c_void_p(0), ks, _ptr(a_log), _ptr(dt_bias),
+             _ptr(seq_of_token), _ptr(cu_seqlens), _ptr(slots), _ptr(q), _ptr(k), _ptr(v), _ptr(gb), T, B, G, H, d, e, _stream()),
+           "dr_conv_prepare")
+
+
+def dr_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: Optional[torch.Tensor], decay: Optional[torch.Tensor],
+            out: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, B: int, H: int, G: int,
+            d: int, e: int, silu: bool = False) -> None:
+    """A walk over every sequence's new tokens with a state S [d, e] a head, float, in `state` [slots, *glr_state_shape]
+    (a view whose slots may be strided).  q, k float views [T, G d], v [T, H e] (rows may be strided; head h reads
+    q/k head h // (H / G)).  With `gb` [T, 2 H] (g | beta) the gated delta rule
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; else with `decay` [H] S <- decay_h S + k v^T.  o = S^T q after
+    the write, into out float [T, H e].  `silu`: q, k, v pass silu on their way in."""
+    _dev("dr_scan", gb, decay, out, cu_seqlens, slots)
+    T = out.shape[0]
+    for name, t, w in (("q", q, G * d), ("k", k, G * d), ("v", v, H * e)):
+        _req(t.is_cuda and t.dtype == torch.float32 and t.shape == (T, w) and t.stride(1) == 1, f"dr_scan: {name} float32 [T, {w}]")
+    _req(T <= 1 or q.stride(0) == k.stride(0), "dr_scan: q and k rows equally far apart")
+    _req((gb is None) != (decay is None), "dr_scan: either g and beta per token or one decay a head")
+    _req(gb is None or (gb.dtype == torch.float32 and gb.shape == (T, 2 * H)), "dr_scan: gb float32 [T, 2 H]")
+    _req(decay is None or (decay.dtype == torch.float32 and decay.numel() == H), "dr_scan: decay float32 [H]")
+    _req(out.dtype == torch.float32 and out.shape == (T, H * e), "dr_scan: out float32 [T, H e]")
+    _req(state.is_cuda and state.dtype == torch.float32 and tuple(state.shape[1:]) == tuple(glr_state_shape(H, d, e))
+         and state[0].is_contiguous(), "dr_scan: state float32 [slots, H, ceil(e/4), rows per lane, 64], every slot's dense")
+    _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "dr_scan: arrays shorter than the batch")
+    _req(H % G == 0 and d <= 512, f"dr_scan: {H} heads over {G} key heads of {d} channels (a multiple; at most 512 channels)")
+    qs = q.stride(0) if T > 1 else G * d
+    vs = v.stride(0) if T > 1 else H * e
+    f = _fn("delta_rule", "br_dr_scan", [_P, _P, c_size_t, _P, c_size_t, _P, c_size_t, _P, _P, _P, c_size_t, _P, _P] + [c_int] * 7 + [_P])
+    _check(f(_ptr(q), _ptr(k), qs, _ptr(v), vs, _ptr(gb), 2 * H, _ptr(decay), _ptr(out), _ptr(state), state.stride(0),
+             _ptr(cu_seqlens), _ptr(slots), B, H, G, d, e, int(gb is not None), int(bool(silu)), _stream()), "dr_scan")
 
 
 def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -878,16 +970,17 @@ def head_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------- routed experts -----
-def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch.Tensor, share: torch.Tensor, top: int) -> None:
+def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch.Tensor, share: torch.Tensor, top: int,
+               out_scale: float = 1.0) -> None:
     """scores float [T, E] (+ bias [E]): the `top` largest per row (ties to the lower number) into chosen int32 [T, top],
-    the softmax over them into share float [T, top]."""
+    the softmax over them times `out_scale` into share float [T, top]."""
     _dev("route_topk", scores, bias, chosen, share)
     T, E = scores.shape
     _req(scores.dtype == torch.float32 and (bias is None or (bias.dtype == torch.float32 and bias.numel() == E)), "route_topk: float32 scores and bias")
     _req(chosen.dtype == torch.int32 and chosen.shape == (T, top) and share.dtype == torch.float32 and share.shape == (T, top), "route_topk: chosen int32 and share float32 [T, top]")
     _req(0 < top <= min(E, 64) and E <= 512, f"route_topk: {top} of {E} experts is outside the kernel's sizes (512 experts, 64 chosen)")
-    f = _fn("routed_experts", "br_route_topk", [_P, _P, _P, _P, c_int, c_int, c_int, _P])
-    _check(f(_ptr(scores), _ptr(bias), _ptr(chosen), _ptr(share), T, E, top, _stream()), "route_topk")
+    f = _fn("routed_experts", "br_route_topk", [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(scores), _ptr(bias), _ptr(chosen), _ptr(share), T, E, top, float(out_scale), _stream()), "route_topk")
 
 
 def experts_up(h: torch.Tensor, w_gu: torch.Tensor, chosen: torch.Tensor, y: torch.Tensor) -> None:

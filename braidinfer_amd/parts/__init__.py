@@ -1,7 +1,7 @@
 from .base import (Part, Norm, NormedInput, ResidualSink, PositionEncoding, RotaryTables, Mixer, MixerContext, FeedForward, Embedding,
                    OutputHead, Runtime, register_part, unregister_part, build_part, block_arrangement,
                    registered_parts)
-from . import norm, rope, attention, pooled_attention, latent_attention, gated_recurrence, time_mix, feedforward, embedding, block  # noqa: F401  (register the built-in parts)
+from . import norm, rope, attention, pooled_attention, latent_attention, gated_recurrence, time_mix, delta_rule, feedforward, embedding, block  # noqa: F401  (register the built-in parts)
 from .linear import linear, fuse_rows
 
 __all__ = ["Part", "Norm", "NormedInput", "ResidualSink", "PositionEncoding", "RotaryTables", "Mixer", "MixerContext", "FeedForward",

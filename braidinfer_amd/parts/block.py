@@ -140,6 +140,48 @@ class ParallelResidual:
             step.probe(f"L{step.schedule_index}.post_ffn", x)
 
 
+class PrenormSideBySide:
+    """x += sum over the layer's mixers of norm_out(mixer(n)) with n = norm(x), then x += feed_forward(norm(x)): several
+    mixers side by side on one normed input (`layer.mixer` and `layer.more_mixers`), each with a norm of its own
+    behind it before the sum.  Roles of `layer.norms`: "mixer" (in front), "mixer_out" for `layer.mixer` and
+    "mixer_out.<role>" for the others (an absent one: the mixer adds into the rows itself), "feed_forward".  A
+    weighting of the sum (a mean, a residual multiplier) is the norms' business (`scale` of an RMS norm).  Each mixer
+    writes float rows of its own; the norm behind it adds the normed rows to the residual rows."""
+
+    def first_norm(self, layer):
+        return None          # the norm's output is kept for all mixers: nothing a product before could prepare in passing
+
+    def run(self, layer, x, step, mixer_ctx) -> None:
+        step.prepared_norm = None
+        dtype = layer.rt.dtype
+        norm = layer.norms.get("mixer")
+        h = x
+        if norm is not None:
+            h = step.ws.get("block_h", tuple(x.shape), dtype)
+            norm.forward(x, h)
+        mixers = ([(None, layer.mixer, mixer_ctx)] if layer.mixer is not None else []) + \
+                 [(role, m, mixer_ctx.others[role]) for role, m in layer.more_mixers.items()]
+        for role, mixer, ctx in mixers:
+            norm_out = layer.norms.get("mixer_out" if role is None else "mixer_out." + role)
+            if norm_out is None:
+                mixer.forward(h, x, step, ctx)
+                continue
+            y = step.ws.get("branch_out", tuple(x.shape), x.dtype)
+            if mixer.through_linear_only:
+                mixer.forward(h, ResidualSink(y, None, overwrite=True), step, ctx)
+            else:
+                y.zero_()
+                mixer.forward(h, y, step, ctx)
+            norm_out.add_normed(y, x)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_mixer", x)
+        if layer.feed_forward is not None:
+            run_residual_branch(layer.feed_forward, layer.norms.get("feed_forward"), step.norm_after_layer, x, step, dtype)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_ffn", x)
+
+
 register_part("block", "prenorm_residual", PrenormResidual, replace=True)
+register_part("block", "prenorm_side_by_side", PrenormSideBySide, replace=True)
 register_part("block", "parallel_residual", ParallelResidual, replace=True)
 register_part("block", "sandwich_residual", SandwichResidual, replace=True)

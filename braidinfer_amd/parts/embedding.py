@@ -40,16 +40,18 @@ class TokenEmbedding(Embedding):
 class LMHead(OutputHead):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, scale: float = 1.0):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, scale: float = 1.0,
+                 tensor: str = "weight"):
         self.V, self.H, self.tied_to, self.scale = int(vocab_size), int(hidden_size), tied_to, float(scale)
+        self.tensor = tensor
         self.weight = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
-        return [] if self.tied_to else [TensorSpec(prefix + "weight", (self.V, self.H))]
+        return [] if self.tied_to else [TensorSpec(prefix + self.tensor, (self.V, self.H))]
 
     def optional_names(self, prefix: str) -> List[str]:
         # a tied checkpoint may still carry a copy of the head
-        return [prefix + "weight"] if self.tied_to else []
+        return [prefix + self.tensor] if self.tied_to else []
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
@@ -61,7 +63,7 @@ class LMHead(OutputHead):
             else:
                 raise WeightError(f"output head: tensor {self.tied_to} is missing", missing=[self.tied_to])
             return
-        name = prefix + "weight"
+        name = prefix + self.tensor
         if name not in tensors:
             raise WeightError(f"output head: tensor {name} is missing", missing=[name])
         self.weight = stream_layout(tensors[name], rt)

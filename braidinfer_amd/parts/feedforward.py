@@ -7,7 +7,8 @@ x += W_d (g sigmoid(alpha g) (u + 1)) + b_d; every projection has a bias, the cl
 the products' float sums.
 
 Routed experts: router scores z = W_r n + b_r in float; a token takes the `top` experts with the largest scores
-(ties to the lower number), weighted by the softmax over those scores only, and x += sum_s share_s expert_s(n)
+(ties to the lower number), weighted by the softmax over those scores only (which is also the softmax over all experts divided by the chosen
+ones' sum), and x += sum_s share_s expert_s(n)
 with an expert W_d (silu(W_g n) * (W_u n)) without biases.  The reference has neither."""
 from __future__ import annotations
 
@@ -116,9 +117,10 @@ class RoutedExperts(FeedForward):
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = True,
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, out_scale: float = 1.0):
         """`names`: "expert" with {e} for the expert's number (the prefix of its three matrices "gate", "up", "down"),
-        "router", "router_bias"."""
+        "router", "router_bias".  `out_scale` multiplies what is added to the residual rows (it rides on the shares)."""
+        self.out_scale = float(out_scale)
         self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(num_experts), int(top)
         if self.I <= 0 or not 0 < self.top <= self.E or self.E > 512 or self.top > 64:
             raise ConfigError(f"routed experts: {top} of {num_experts} experts of inner width {intermediate_size} "
@@ -167,7 +169,7 @@ class RoutedExperts(FeedForward):
         linear(h, self.w_router, scores, step.ws)
         chosen = step.ws.get("moe_chosen", (T, self.top), torch.int32)
         share = step.ws.get("moe_share", (T, self.top), torch.float32)
-        K.route_topk(scores, self.b_router, chosen, share, self.top)
+        K.route_topk(scores, self.b_router, chosen, share, self.top, self.out_scale)
         few = step.is_decode or T < int(os.environ.get("BRAIDINFER_BY_EXPERT_FROM", str(self.BY_EXPERT_FROM)))
         if few and not K.experts_grouped_takes(dt, self.H, self.I):
             # every pair reads its expert's rows itself: the 32-bit path, and widths the grouped kernels do not take

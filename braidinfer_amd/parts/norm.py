@@ -1,5 +1,8 @@
 """RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, plain `w` (reference: op_rmsnorm_wx,
-kernels/megakernel_ops.hip:862-904; eps default and key in config.rs:249-252).
+kernels/megakernel_ops.hip:862-904; eps default and key in config.rs:249-252).  A checkpoint that stores the weight
+around zero names an `offset` (w = offset + stored), and a norm whose output is always multiplied by a constant
+(a branch's share of a sum, a residual multiplier) names it as `scale`; both are folded into the kept float weight
+at load.
 
 LayerNorm: y = (x - mean) / sqrt(var + eps) * w, var the mean of the squared deviations, a weight
 and no bias (absent in the reference, whose models norm without centering).
@@ -20,16 +23,22 @@ from .base import Norm, ProductRuns, Runtime, register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+    def __init__(self, size: int, eps: float, tensor: str = "weight", offset: float = 0.0, scale: float = 1.0):
         self.size, self.eps, self.tensor = int(size), float(eps), tensor
+        self.offset, self.scale = float(offset), float(scale)
         self.weight: Optional[torch.Tensor] = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(prefix + self.tensor, (self.size,), kind="vector", init="ones")]
+        return [TensorSpec(prefix + self.tensor, (self.size,), kind="vector", init="ones" if self.offset == 0.0 else "normal")]
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = rt.own(tensors[prefix + self.tensor].to(torch.float32))
+        w = tensors[prefix + self.tensor].to(torch.float32)
+        if self.offset != 0.0:
+            w = w + self.offset
+        if self.scale != 1.0:
+            w = w * self.scale
+        self.weight = rt.own(w)
 
     def forward(self, x, out, rows=None):
         K.rmsnorm(x, self.weight, out, self.eps, rows)

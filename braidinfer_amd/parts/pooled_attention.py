@@ -11,6 +11,14 @@ them.  Tokens that left the window and whose block is not complete behind it are
 Tokens and blocks share one softmax of the scores (q . k) * scale, which may carry a sink: a key
 of score 0 without a value, i.e. one added to the denominator.  Key and value widths may differ.
 
+Without a window (`window` None) every earlier token is seen: plain causal attention through the same kernels.
+Further options, each a parameter: the values may be the keys as projected, before their norm (`values_from_keys`,
+no value matrix); the query/key norm may go without weights (`qk_norm_weights` False); the query may be multiplied
+by a temperature that grows with the logarithm of the position, 1 + c ln(floor((p + 1) / n) + 1) (`q_temp` = (c, n));
+the heads' outputs may pass a sigmoid gate projected from the mixer's input, one number per output element or one
+per head (`gate` "element" / "head"), before the output projection; `out_scale` multiplies what the mixer adds to the
+residual rows (it rides on the gate, or on the output matrix where there is none).
+
 Cache: the mixer's own unit keeps the tokens' rows as long as a later query or a block that is
 not pooled yet needs them (`CacheNeed.live_from`); a further unit under the role "pooled" keeps
 one row per block (`CacheNeed.tokens_per_row`).  Scores, softmax weights, norms and angles are
@@ -52,7 +60,8 @@ class PooledWindowAttention(Mixer):
     graph_safe = True
     through_linear_only = True
 
-    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+    NO_WINDOW = 1 << 30          # the kernels' window when every earlier token is seen: beyond any position
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "gate": "g_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
              "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
 
@@ -60,20 +69,33 @@ class PooledWindowAttention(Mixer):
                  window: int, pool: int = 0, scale: Optional[float] = None, sink: bool = False, bias: bool = False,
                  qk_norm_eps: Optional[float] = None, position: Optional[str] = None,
                  value_mix: Optional[str] = None, value_mix_group: str = "v_first",
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, values_from_keys: bool = False, qk_norm_weights: bool = True,
+                 q_temp=None, gate: Optional[str] = None, out_scale: float = 1.0):
         """`qk_norm_eps` None: no query/key norm.  `value_mix`: None, "source" (this layer's values are what
         later layers of the same `value_mix_group` mix with; its own scalar is loaded and unused) or "mix"."""
         if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
             raise ConfigError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if not 0 < key_dim <= MAX_WIDTH or not 0 < value_dim <= MAX_WIDTH:
             raise ConfigError(f"attention: head widths {key_dim} (keys) and {value_dim} (values) must lie in 1..{MAX_WIDTH}")
-        if window is None or int(window) <= 0 or int(pool or 0) < 0:
-            raise ConfigError(f"attention: the window must be positive and the pooled block's size not negative, got {window}, {pool}")
+        if (window is not None and int(window) <= 0) or int(pool or 0) < 0 or (window is None and pool):
+            raise ConfigError(f"attention: the window must be positive (or None: all earlier tokens, no pooled blocks) and the "
+                              f"pooled block's size not negative, got {window}, {pool}")
+        if gate not in (None, "element", "head"):
+            raise ConfigError(f"attention: gate must be None, 'element' or 'head', got {gate!r}")
+        if values_from_keys and (key_dim != value_dim or bias or value_mix is not None):
+            raise ConfigError("attention: values taken from the keys have the keys' width, no bias and no mixing")
+        if q_temp is not None and (len(q_temp) != 2 or int(q_temp[1]) <= 0):
+            raise ConfigError(f"attention: q_temp is (coefficient, positions a step > 0), got {q_temp!r}")
         if value_mix not in (None, "source", "mix"):
             raise ConfigError(f"attention: value_mix must be None, 'source' or 'mix', got {value_mix!r}")
         self.H, self.nq, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.dk, self.dv = int(key_dim), int(value_dim)
-        self.window, self.pool = int(window), int(pool or 0)
+        self.full = window is None
+        self.window, self.pool = (self.NO_WINDOW if window is None else int(window)), int(pool or 0)
+        self.values_from_keys, self.qk_norm_weights = bool(values_from_keys), bool(qk_norm_weights)
+        self.q_temp = None if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+        self.gate, self.out_scale = gate, float(out_scale)
+        self.n_gate = 0 if gate is None else (self.nq if gate == "head" else self.nq * self.dv)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
         self.sink, self.bias = bool(sink), bool(bias)
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
@@ -93,10 +115,13 @@ class PooledWindowAttention(Mixer):
         out.append(TensorSpec(prefix + n["k"], (self.nkv * self.dk, self.H)))
         if self.bias:
             out.append(TensorSpec(prefix + n["k_bias"], (self.nkv * self.dk,), kind="vector", init="normal"))
-        out.append(TensorSpec(prefix + n["v"], (self.nkv * self.dv, self.H)))
+        if not self.values_from_keys:
+            out.append(TensorSpec(prefix + n["v"], (self.nkv * self.dv, self.H)))
         if self.bias:
             out.append(TensorSpec(prefix + n["v_bias"], (self.nkv * self.dv,), kind="vector", init="normal"))
-        if self.qk_norm_eps is not None:
+        if self.gate is not None:
+            out.append(TensorSpec(prefix + n["gate"], (self.n_gate, self.H)))
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             out += [TensorSpec(prefix + n["q_norm"], (self.dk,), kind="vector", init="ones"),
                     TensorSpec(prefix + n["k_norm"], (self.dk,), kind="vector", init="ones")]
         if self.value_mix is not None:
@@ -107,18 +132,30 @@ class PooledWindowAttention(Mixer):
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
         n = self.names
-        self.w_qkv = fused_layout([tensors[prefix + n[x]] for x in ("q", "k", "v")], rt)
-        self.w_o = stream_layout(tensors[prefix + n["o"]], rt)
+        # one product for all projections of the mixer's input: q | k | v (unless the keys serve) | gate
+        mats = ["q", "k"] + ([] if self.values_from_keys else ["v"]) + (["gate"] if self.gate is not None else [])
+        self.w_qkv = fused_layout([tensors[prefix + n[x]] for x in mats], rt)
+        self.gate_col0 = self.nq * self.dk + self.nkv * self.dk + (0 if self.values_from_keys else self.nkv * self.dv)
+        w_o = tensors[prefix + n["o"]]
+        if self.gate is None and self.out_scale != 1.0:          # no gate to carry the multiplier: the matrix does
+            w_o = (w_o.to(torch.float32) * self.out_scale).to(w_o.dtype)
+        self.w_o = stream_layout(w_o, rt)
         if self.bias:
             self.b_qkv = rt.own(torch.cat([tensors[prefix + n[x]].to(torch.float32).reshape(-1) for x in ("q_bias", "k_bias", "v_bias")]))
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             self.q_norm = rt.own(tensors[prefix + n["q_norm"]].to(torch.float32))
             self.k_norm = rt.own(tensors[prefix + n["k_norm"]].to(torch.float32))
+        elif self.qk_norm_eps is not None:
+            ones = rt.empty((self.dk,), torch.float32)
+            ones.fill_(1.0)
+            self.q_norm = self.k_norm = ones
         if self.value_mix == "mix":
             self.mix = rt.own(tensors[prefix + n["value_mix"]].to(torch.float32).reshape(1))
 
     # ---- what it keeps -----------------------------------------------------------------
     def cache_need(self) -> CacheNeed:
+        if self.full:
+            return CacheNeed(kv_heads=self.nkv, head_dim=self.dk, value_dim=self.dv)
         return CacheNeed(kv_heads=self.nkv, head_dim=self.dk, value_dim=self.dv,
                          live_from=window_and_open_block(self.window, self.pool))
 
@@ -152,7 +189,7 @@ class PooledWindowAttention(Mixer):
         if ctx.storage is None or (self.pool and "pooled" not in ctx.others):
             raise StepError("attention: the run order gave this mixer no cache unit (or none for its pooled rows)")
         # the projections' float sums: norms and angles work on them before anything is rounded
-        qkv = step.ws.get("pwa_qkv", (T, nq * dk + nkv * (dk + dv)), torch.float32)
+        qkv = step.ws.get("pwa_qkv", (T, self.gate_col0 + self.n_gate), torch.float32)
         linear(h, self.w_qkv, qkv, step.ws)
         q = step.ws.get("pwa_q", (T, nq * dk), dt)
         v_first, role = None, 0
@@ -172,7 +209,8 @@ class PooledWindowAttention(Mixer):
         K.pwa_prepare(qkv, self.b_qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
                       tables.cos if tables else None, tables.sin if tables else None, tables.rotary_dim if tables else 0,
                       step.positions, step.seq_of_token, step.slots, ctx.block_table, q, unit, v_first, self.mix, role,
-                      nq, nkv, dk, dv, ctx.page_tokens, ctx.writes_cache)
+                      nq, nkv, dk, dv, ctx.page_tokens, ctx.writes_cache, self.values_from_keys,
+                      self.q_temp[0] if self.q_temp else 0.0, self.q_temp[1] if self.q_temp else 0)
         pooled = ctx.others.get("pooled")
         if pooled is not None and ctx.writes_cache:
             K.pwa_pool(unit, ctx.block_table, pooled.storage, pooled.block_table, step.cu_seqlens, step.ctx_lens, step.slots,
@@ -193,6 +231,8 @@ class PooledWindowAttention(Mixer):
             # the 32-bit path and other sizes: four waves per (query, head) in float
             K.pwa_attend(q, o, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit, p_table, p_unit,
                          nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
+        if self.gate is not None:
+            K.pwa_gate(o, qkv[:, self.gate_col0:], nq, dv, self.gate == "head", self.out_scale)
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
 

@@ -23,6 +23,7 @@ import torch
 
 from .. import kernels as K
 from ..errors import ConfigError, StepError
+from ..weights import TensorSpec
 from .base import PositionEncoding, RotaryTables, Runtime, register_part
 
 
@@ -97,5 +98,36 @@ class NoPositionEncoding(PositionEncoding):
         self.rt = rt
 
 
+class LearnedPositions(PositionEncoding):
+    """A learnt vector per position, added to the embeddings (not scaled): x[t] += table[p_t].  The table has `rows`
+    positions; a step that reaches beyond it is refused.  `tensor` is the piece of the table's name behind the part's
+    prefix.  The mixers see nothing of it (`gives` "embedding")."""
+    graph_safe = True
+    gives = "embedding"
+
+    def __init__(self, rows: int, hidden_size: int, tensor: str = "weight"):
+        self.rows, self.H, self.tensor = int(rows), int(hidden_size), tensor
+        self.table = None
+
+    def weight_specs(self, prefix: str):
+        return [TensorSpec(prefix + self.tensor, (self.rows, self.H))]
+
+    def load(self, tensors, prefix, rt):
+        self.rt = rt
+        self.table = rt.own(tensors[prefix + self.tensor])
+
+    def add_to_embedding(self, x, step) -> None:
+        if step.position_ids.dim() != 1:
+            raise StepError("learnt positions take one position number a token")
+        if step.position_ids is step.positions:
+            # a recorded single-token step carries no host lengths (its slots read -1): there the kernel adds
+            # nothing for a position outside the table
+            longest = max((s + n for s, n, slot in zip(step.host_start, step.host_new, step.host_slots) if slot >= 0), default=0)
+            if longest > self.rows:
+                raise StepError(f"a sequence of {longest} tokens is beyond the model's {self.rows} learnt positions")
+        K.add_position_rows(x, self.table, step.position_ids)
+
+
+register_part("position", "learned", LearnedPositions, replace=True)
 register_part("position", "rope", RotaryEncoding, replace=True)
 register_part("position", "none", NoPositionEncoding, replace=True)
