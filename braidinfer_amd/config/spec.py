@@ -120,6 +120,8 @@ class ModelSpec:
     bos_token_id: Optional[int] = None
     # tensor-name prefix of a position encoding's tensors, by the encoding's name (absent: "position.<name>.")
     position_prefixes: Dict[str, str] = field(default_factory=dict)
+    # tensors a checkpoint may carry that no part reads (a norm in front of a feed-forward the layer does not have)
+    optional_tensors: List[str] = field(default_factory=list)
 
 
 def default_schedule(n_layers: int) -> List[ScheduleEntry]:

@@ -236,7 +236,8 @@ def build_spec(cfg: ZivovikConfig) -> ModelSpec:
         positions={"learned": PartSpec("learned", {"rows": cfg.max_positions, "hidden_size": W, "tensor": ""})},
         max_position_embeddings=cfg.max_positions,
         embedding_prefix="embed", final_norm_prefix="final.norm", lm_head_prefix="head",
-        stop_token_ids=[], bos_token_id=None, position_prefixes={"learned": "pos"})
+        stop_token_ids=[], bos_token_id=None, position_prefixes={"learned": "pos"},
+        optional_tensors=[f"l{i}.norm2" for i, l in enumerate(cfg.layers) if l.get("mlp") is None])
 
 
 def _attention(heads, kv_heads, dim, coef=0.4, every=128):

@@ -153,7 +153,7 @@ class DecoderModel:
         return out
 
     def optional_names(self) -> List[str]:
-        out: List[str] = []
+        out: List[str] = list(self.spec.optional_tensors)
         for part, prefix in self._named_parts():
             f = getattr(part, "optional_names", None)
             if f:
