@@ -74,7 +74,8 @@ LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_
              "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16", "pwa_decode_bf16",
              "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax", "wkv_scan", "wkv_scan_pieces", "shift_mix", "head_norm_gate", "tanh",
              "latent_prepare", "head_linear", "route_topk", "experts_up", "experts_down", "experts_sort", "experts_gather",
-             "experts_combine", "experts_up_grouped", "experts_down_grouped", "experts_gemm", "clamped_glu", "add_bias_rows"]
+             "experts_combine", "experts_up_grouped", "experts_down_grouped", "experts_gemm", "clamped_glu", "add_bias_rows",
+             "add_position_rows", "pwa_gate", "dr_conv_prepare", "dr_scan"]
 
 
 def kernel_share(torch, eng, entries_of, classes):
@@ -263,7 +264,10 @@ class Shape:
 # single-token step of each (run eagerly, bracketed by events).  `--design sidirax`: the Sidirax design beside
 # Kesitar (the library's closest model: attention layers between linear recurrences, a sink in the softmax) at
 # equal width and layers; what is set beside a design is a Mistral configuration (a dict) or a preset's name.
+# `--design zivovik`: the Zivovik design beside Sidirax (the library's closest model: attention layers between
+# recurrences over an outer-product state, routed experts) at equal width and number of layer runs.
 DESIGN_SIZES = {
+    "zivovik": {"1b": ("zivovik-1b", "sidirax-1b"), "7b": ("zivovik-7b", "sidirax-7b")},
     "sidirax": {"1b": ("sidirax-1b", "kesitar-1b"), "7b": ("sidirax-7b", "kesitar-7b")},
     "kesitar": {
         "1b": ("kesitar-1b", dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
@@ -393,7 +397,7 @@ def design_comparison(args) -> int:
     import torch
     import braidinfer_amd as B
     sizes = DESIGN_SIZES[args.design]
-    beside = "kesitar" if args.design == "sidirax" else "mistral"
+    beside = {"sidirax": "kesitar", "zivovik": "sidirax"}.get(args.design, "mistral")
     line = {"metric": f"{args.design} beside {beside} at equal size: prefill and decode tokens/s, bf16, random weights",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "layers": args.layers or 8,
             "steps": args.steps, "warmup": args.warmup, "sizes": {}}
@@ -445,7 +449,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true",
                     help="skip the further batch sizes, prompt lengths and workloads, the measured peaks and the kernel shares")
     ap.add_argument("--design", default=None, choices=sorted(DESIGN_SIZES),
-                    help="instead of the workload: this design beside Mistral at equal size (prefill, decode, kernel times)")
+                    help="instead of the workload: this design beside its closest model at equal size (prefill, decode, kernel times)")
     ap.add_argument("--design-size", default=None, help="sizes of --design to run, with commas (default: all)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the prefill of --prefill-tokens (for profiles); prints its own line")

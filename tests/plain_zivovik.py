@@ -79,7 +79,7 @@ def unit_vectors(x):
     return x / np.sqrt((x * x).sum(axis=-1, keepdims=True) + 1e-6)
 
 
-def delta_rule(q, k, v, beta, g):
+def delta_rule(q, k, v, beta, g, return_state=False):
     """One head: q, k [T, d], v [T, e], beta, g [T].  S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q."""
     T, d = q.shape
     S = np.zeros((d, v.shape[1]))
@@ -89,10 +89,10 @@ def delta_rule(q, k, v, beta, g):
         u = beta[t] * (v[t] - S.T @ k[t])
         S = S + np.outer(k[t], u)
         o[t] = S.T @ q[t]
-    return o
+    return (o, S) if return_state else o
 
 
-def decayed_outer_sum(q, k, v, decay):
+def decayed_outer_sum(q, k, v, decay, return_state=False):
     """One head with a fixed decay: S_t = decay S_(t-1) + k_t v_t^T, o_t = S_t^T q_t."""
     T, d = q.shape
     S = np.zeros((d, v.shape[1]))
@@ -100,7 +100,7 @@ def decayed_outer_sum(q, k, v, decay):
     for t in range(T):
         S = decay * S + np.outer(k[t], v[t])
         o[t] = S.T @ q[t]
-    return o
+    return (o, S) if return_state else o
 
 
 # ------------------------------------------------------------------ mixers ----------
@@ -169,14 +169,14 @@ def lightning_mixer(h, w, p, m, eps):
 def routed_ff(h, w, p, mlp, margins=None):
     """Scores are the softmax of the router's logits over all experts; the `top` largest are chosen and weighted by their
     scores over the chosen scores' sum.  `margins` (a list) receives, per token, the gap between the last chosen and the
-    first left-out score."""
+    first left-out router logit."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     z = h @ w[p + "router"].T
     s = np.exp(z - z.max(axis=1, keepdims=True))
     s = s / s.sum(axis=1, keepdims=True)
     order = np.argsort(-s, axis=1, kind="stable")
     if margins is not None and top < E:
-        srt = np.take_along_axis(s, order, axis=1)
+        srt = np.take_along_axis(z, order, axis=1)
         margins.append(srt[:, top - 1] - srt[:, top])
     out = np.zeros((h.shape[0], w[p + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
@@ -306,7 +306,8 @@ def random_weights(cfg, seed, gain=1.0, router_gain=1.0):
 
     def attention(q, m, own_values, gate_rows):
         H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-        w[q + "q"], w[q + "k"] = mat(H * d, W, 2.0 * gain), mat(G * d, W, 2.0 * gain)
+        g = gain if own_values else 2.0 * gain          # queries and keys that pass no norm set the softmax's sharpness themselves
+        w[q + "q"], w[q + "k"] = mat(H * d, W, g), mat(G * d, W, g)
         if own_values:
             w[q + "v"] = mat(G * e, W)
         w[q + "g"], w[q + "o"] = mat(gate_rows, W), mat(W, H * e)
