@@ -31,18 +31,21 @@ __device__ __forceinline__ float dr_silu(float z) { return z / (1.0f + expf(-z))
 
 // ------------------------------------------------------------------- prepare -------
 // rows [T, width] float, the projections' sums: q (G heads of d) | k (G of d) | v (H of e) | b (H) | a (H) | ...
-// One wave per (token, head row) with head rows = G query heads, G key heads, H value heads.  Channel ch of the
+// One wave per (token, head row) with head rows = G query heads, G key heads, H value heads; four waves a workgroup.  Channel ch of the
 // C = 2 G d + H e convolved channels is column ch of `rows`; taps [C, n] float, the last column the current token's;
 // `kept` holds per slot the last n - 1 inputs of every channel, [n - 1][C] (zeros in a new slot).
 // Out: qo, ko [T, G d] (silu, unit length per head, q times d^-1/2), vo [T, H e] (silu), gb [T, 2 H]:
 // g = exp(-exp(A_log) softplus(a + dt_bias)) then beta = sigmoid(b).
-__global__ __launch_bounds__(64) void dr_conv_prepare_kernel(
+__global__ __launch_bounds__(256) void dr_conv_prepare_kernel(
     const float* __restrict__ rows, int width, const float* __restrict__ taps, int n_taps,
     const float* __restrict__ kept, size_t kept_stride, const float* __restrict__ a_log,
     const float* __restrict__ dt_bias, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, float* __restrict__ qo, float* __restrict__ ko, float* __restrict__ vo,
-    float* __restrict__ gb, int G, int H, int d, int e) {
-    const int t = blockIdx.x, hr = blockIdx.y, lane = threadIdx.x;
+    float* __restrict__ gb, int T, int G, int H, int d, int e) {
+    const int n_hr = 2 * G + H;
+    const long long unit = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);          // a wave a (token, head row)
+    if (unit >= (long long)T * n_hr) return;
+    const int t = (int)(unit / n_hr), hr = (int)(unit - (long long)t * n_hr), lane = threadIdx.x & 63;
     const bool is_q = hr < G, is_k = !is_q && hr < 2 * G;
     const int head = is_q ? hr : (is_k ? hr - G : hr - 2 * G);
     const int n = (is_q || is_k) ? d : e;
@@ -117,11 +120,13 @@ extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* tap
     if (T <= 0 || B <= 0) return BR_OK;
     const long long C = 2LL * G * d + (long long)H * e;
     if (G <= 0 || H <= 0 || H % G || d <= 0 || e <= 0 || d > 64 * DR_MAX_EPL || e > 64 * DR_MAX_EPL || n_taps < 1 ||
-        n_taps > DR_MAX_TAPS || width < C + 2 * H || 2 * G + H > 65535 || B > 65535 || (C + 255) / 256 > 65535 ||
+        n_taps > DR_MAX_TAPS || width < C + 2 * H || ((long long)T * (2 * G + H) + 3) / 4 > 0x7fffffffLL || B > 65535 ||
+        (C + 255) / 256 > 65535 ||
         (n_taps > 1 && (!kept || kept_stride < (size_t)(n_taps - 1) * C)) || !a_log || !dt_bias)
         return BR_BAD_ARG;
-    dr_conv_prepare_kernel<<<dim3(T, 2 * G + H), 64, 0, s>>>(rows, width, taps, n_taps, kept, kept_stride, a_log, dt_bias,
-                                                            seq_of_token, cu_seqlens, slots, qo, ko, vo, gb, G, H, d, e);
+    const unsigned blocks = (unsigned)(((long long)T * (2 * G + H) + 3) / 4);
+    dr_conv_prepare_kernel<<<blocks, 256, 0, s>>>(rows, width, taps, n_taps, kept, kept_stride, a_log, dt_bias, seq_of_token,
+                                                 cu_seqlens, slots, qo, ko, vo, gb, T, G, H, d, e);
     int rc = br_check_launch();
     if (rc != BR_OK || n_taps == 1) return rc;
     dr_conv_keep_kernel<<<dim3(B, (unsigned)((C + 255) / 256)), 256, 0, s>>>(rows, width, n_taps, kept, kept_stride, cu_seqlens,
@@ -135,7 +140,9 @@ extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* tap
 // head from `gb` (rows `gb_stride` apart, g at [h], beta at [H + h]); else the head's one decay `g_head[h]` and
 // u = v.  SILU: q, k and v are the projections' float sums and pass silu on their way into LDS.
 // grid (sequences, heads, ceil(e / 16)), 256 threads; a slot's state as `glr_state_shape` says.
-template <int RPL, int TC, bool DELTA, bool SILU>
+// LOCAL (the first pass over a long prompt cut into pieces, see `br_dr_scan_pieces`): the state starts at zero, nothing
+// is written to o, and the last state goes to the piece's scratch.
+template <int RPL, int TC, bool DELTA, bool SILU, bool LOCAL>
 __global__ __launch_bounds__(256) void dr_scan_kernel(
     const float* __restrict__ q, const float* __restrict__ k, size_t qk_stride, const float* __restrict__ v,
     size_t v_stride, const float* __restrict__ gb, size_t gb_stride, const float* __restrict__ g_head,
@@ -158,14 +165,14 @@ __global__ __launch_bounds__(256) void dr_scan_kernel(
     const bool live = c < e;
     const int he = H * e;
     if (slot < 0) {                                // padding: no state behind it; its rows of o are zero
-        if (g == 0 && live) for (int t = t0; t < t1; ++t) o[(size_t)t * he + h * e + c] = 0.f;
+        if (!LOCAL && g == 0 && live) for (int t = t0; t < t1; ++t) o[(size_t)t * he + h * e + c] = 0.f;
         return;
     }
     const int ncb4 = (e + 3) >> 2;
     float* S = state + (size_t)slot * slot_stride + (((size_t)h * ncb4 + cb4) * RPL) * 64 + lane;
     float st[RPL];
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) st[r] = cb4 < ncb4 ? S[(size_t)r * 64] : 0.f;
+    for (int r = 0; r < RPL; ++r) st[r] = (!LOCAL && cb4 < ncb4) ? S[(size_t)r * 64] : 0.f;
     const float g_fixed = DELTA ? 1.f : g_head[h];
     int l_tt[NL], l_r4[NL];
 #pragma unroll
@@ -262,7 +269,7 @@ __global__ __launch_bounds__(256) void dr_scan_kernel(
                 }
             }
             sum = dr_row16_sum(sum);
-            if (g == 0 && live) orow[0] = sum;
+            if (!LOCAL && g == 0 && live) orow[0] = sum;
             orow += he;
         }
         if (more) stage(buf ^ 1);
@@ -280,25 +287,24 @@ static inline int dr_rpl(int d) {
     return r <= 4 ? 4 : (r <= 8 ? 8 : (r <= 16 ? 16 : 32));
 }
 
-// `delta` 1: the gated delta rule with `gb`; 0: the decayed outer sum with `g_head`.  `silu` 1: q, k, v pass silu.
-extern "C" int br_dr_scan(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride, const float* gb,
+template <bool LOCAL>
+static int dr_scan_launch(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride, const float* gb,
                           size_t gb_stride, const float* g_head, float* o, float* state, size_t slot_stride,
                           const int* cu_seqlens, const int* slots, int B, int H, int G, int d, int e, int delta, int silu,
                           hipStream_t s) {
-    if (B <= 0) return BR_OK;
     const int ncb4 = (e + 3) / 4, rpl = dr_rpl(d);
-    if (H <= 0 || H > 65535 || G <= 0 || H % G || d <= 0 || e <= 0 || d > 512 || (e + 15) / 16 > 65535 ||
+    if (H <= 0 || H > 65535 || G <= 0 || H % G || d <= 0 || e <= 0 || d > 512 || (e + 15) / 16 > 65535 || B > 0x7fffffff ||
         qk_stride < (size_t)G * d || v_stride < (size_t)H * e || slot_stride < (size_t)H * ncb4 * rpl * 64 ||
-        (delta && (!gb || gb_stride < (size_t)2 * H)) || (!delta && !g_head))
+        (delta && (!gb || gb_stride < (size_t)2 * H)) || (!delta && !g_head) || (LOCAL && delta))
         return BR_BAD_ARG;
     dim3 grid(B, H, (e + 15) / 16);
 #define DR_GO(R, TC, D, A) do { \
         const size_t lds = (size_t)(4 * TC * R * 16 + 2 * TC * 16 + 2 * TC * 2) * sizeof(float); \
-        dr_scan_kernel<R, TC, D, A><<<grid, 256, lds, s>>>(q, k, qk_stride, v, v_stride, gb, gb_stride, g_head, o, state, slot_stride, \
-                                                          cu_seqlens, slots, H, G, d, e); \
+        dr_scan_kernel<R, TC, D, A, LOCAL><<<grid, 256, lds, s>>>(q, k, qk_stride, v, v_stride, gb, gb_stride, g_head, o, state, slot_stride, \
+                                                                 cu_seqlens, slots, H, G, d, e); \
     } while (0)
 #define DR_SCAN(R, TC) do { \
-        if (delta) { if (silu) DR_GO(R, TC, true, true); else DR_GO(R, TC, true, false); } \
+        if (delta) { if (LOCAL) return BR_BAD_ARG; if (silu) DR_GO(R, TC, true, true); else DR_GO(R, TC, true, false); } \
         else { if (silu) DR_GO(R, TC, false, true); else DR_GO(R, TC, false, false); } \
     } while (0)
     if (rpl == 4) DR_SCAN(4, 16);
@@ -308,4 +314,66 @@ extern "C" int br_dr_scan(const float* q, const float* k, size_t qk_stride, cons
 #undef DR_SCAN
 #undef DR_GO
     return br_check_launch();
+}
+
+// `delta` 1: the gated delta rule with `gb`; 0: the decayed outer sum with `g_head`.  `silu` 1: q, k, v pass silu.
+extern "C" int br_dr_scan(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride, const float* gb,
+                          size_t gb_stride, const float* g_head, float* o, float* state, size_t slot_stride,
+                          const int* cu_seqlens, const int* slots, int B, int H, int G, int d, int e, int delta, int silu,
+                          hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    return dr_scan_launch<false>(q, k, qk_stride, v, v_stride, gb, gb_stride, g_head, o, state, slot_stride, cu_seqlens, slots,
+                                 B, H, G, d, e, delta, silu, s);
+}
+
+// Between the two passes over a prompt cut into `pieces` pieces per sequence, for the decayed outer sum: from the
+// sequence's own state s_0 and every piece's local last state L_c, the state each piece starts from,
+// s_(c+1) = decay_h^(tokens of piece c) s_c + L_c, written over L_c; the last one becomes the sequence's state.
+// grid (sequences, heads * column blocks of 4), block 64.
+__global__ __launch_bounds__(64) void dr_carry_kernel(float* __restrict__ state, size_t slot_stride, const int* __restrict__ slots,
+                                                      float* __restrict__ piece_state, size_t piece_stride,
+                                                      const int* __restrict__ piece_cu, const float* __restrict__ g_head,
+                                                      int pieces, int ncb4, int rpl) {
+    const int b = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x;
+    const int slot = slots[b];
+    if (slot < 0) return;
+    const float decay = g_head[hc / ncb4];
+    for (int k = 0; k < rpl; ++k) {
+        const size_t idx = ((size_t)hc * rpl + k) * 64 + lane;
+        float sv = state[(size_t)slot * slot_stride + idx];
+        for (int c = 0; c < pieces; ++c) {
+            const size_t v = (size_t)b * pieces + c;
+            const float local = piece_state[v * piece_stride + idx];
+            piece_state[v * piece_stride + idx] = sv;
+            sv = fmaf(powf(decay, (float)(piece_cu[v + 1] - piece_cu[v])), sv, local);
+        }
+        state[(size_t)slot * slot_stride + idx] = sv;
+    }
+}
+
+// The decayed outer sum over a step of long prompts with every sequence cut into `pieces` pieces that run side by side:
+// the recurrence is linear in the state, so a piece can be walked from a zero state first (its last state L), the
+// pieces' true first states follow from s_(c+1) = decay^n_c s_c + L_c, and a second walk from those writes o.  Twice
+// the arithmetic for `pieces` times the workgroups; results differ from the plain walk by the rounding of that one
+// combination per piece.  `piece_cu` [B * pieces + 1] cuts the packed tokens (pieces of a sequence in order, empty
+// ones allowed), `piece_slots` [B * pieces] is the piece's own number (or -1 for a padding sequence's),
+// `piece_state` [B * pieces][state of a slot] is scratch.
+extern "C" int br_dr_scan_pieces(const float* q, const float* k, size_t qk_stride, const float* v, size_t v_stride,
+                                 const float* g_head, float* o, float* state, size_t slot_stride, const int* slots,
+                                 const int* piece_cu, const int* piece_slots, float* piece_state, int B, int pieces, int H,
+                                 int d, int e, int silu, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (pieces <= 0 || (long long)B * pieces > 65535 || B > 65535) return BR_BAD_ARG;
+    const int ncb4 = (e + 3) / 4, rpl = dr_rpl(d);
+    const size_t piece_stride = (size_t)H * ncb4 * rpl * 64;
+    int rc = dr_scan_launch<true>(q, k, qk_stride, v, v_stride, nullptr, 0, g_head, o, piece_state, piece_stride, piece_cu,
+                                  piece_slots, B * pieces, H, H, d, e, 0, silu, s);
+    if (rc != BR_OK) return rc;
+    if ((long long)H * ncb4 > 65535 || slot_stride < piece_stride) return BR_BAD_ARG;
+    dr_carry_kernel<<<dim3(B, H * ncb4), 64, 0, s>>>(state, slot_stride, slots, piece_state, piece_stride, piece_cu, g_head, pieces,
+                                                     ncb4, rpl);
+    rc = br_check_launch();
+    if (rc != BR_OK) return rc;
+    return dr_scan_launch<false>(q, k, qk_stride, v, v_stride, nullptr, 0, g_head, o, piece_state, piece_stride, piece_cu,
+                                 piece_slots, B * pieces, H, H, d, e, 0, silu, s);
 }

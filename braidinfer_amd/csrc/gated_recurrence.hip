@@ -658,11 +658,43 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
     }
 }
 
+// The same for rows of many channels (all heads normed together, say): a workgroup a (token, head) row.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                                  const float* __restrict__ gate, size_t gate_stride,
+                                                                  T* __restrict__ y, int H, int e, float eps, int gate_sigmoid) {
+    __shared__ float scratch[16];
+    const size_t r = blockIdx.x;
+    const float* orow = o + r * e;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < e; i += 256) { const float v = orow[i]; ss = fmaf(v, v, ss); }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)e + eps);
+    const size_t t = r / H;
+    const int hh = (int)(r - t * H);
+    const float* grow = gate ? gate + t * gate_stride + (size_t)hh * e : nullptr;
+    const float* wrow = w ? w + (size_t)hh * e : nullptr;
+    T* yrow = y + r * e;
+    for (int i = threadIdx.x; i < e; i += 256) {
+        float v = orow[i] * inv;
+        if (wrow) v *= wrow[i];
+        if (grow) { const float z = grow[i]; v *= (gate_sigmoid ? 1.0f : z) / (1.0f + expf(-z)); }
+        yrow[i] = from_f32<T>(v);
+    }
+}
+
+#define HNG_WIDE_FROM 512      // channels of a row from which a workgroup takes it
+
 extern "C" int br_head_norm_gate(const float* o, const float* w, const float* gate, size_t gate_stride, void* y, int y_is_bf16,
                                  int T, int H, int e, float eps, int gate_sigmoid, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (H <= 0 || e <= 0 || (gate && gate_stride < (size_t)H * e)) return BR_BAD_ARG;
     const size_t n_rows = (size_t)T * H;
+    if (e >= HNG_WIDE_FROM) {
+        if (n_rows > 0x7fffffffULL) return BR_BAD_ARG;
+        if (y_is_bf16) head_norm_gate_wide_kernel<bf16><<<(unsigned)n_rows, 256, 0, s>>>(o, w, gate, gate_stride, (bf16*)y, H, e, eps, gate_sigmoid);
+        else head_norm_gate_wide_kernel<float><<<(unsigned)n_rows, 256, 0, s>>>(o, w, gate, gate_stride, (float*)y, H, e, eps, gate_sigmoid);
+        return br_check_launch();
+    }
     const unsigned blocks = (unsigned)((n_rows + 15) / 16);
     if (y_is_bf16) head_norm_gate_kernel<bf16><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (bf16*)y, n_rows, H, e, eps, gate_sigmoid);
     else head_norm_gate_kernel<float><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (float*)y, n_rows, H, e, eps, gate_sigmoid);

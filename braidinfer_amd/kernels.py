@@ -917,6 +917,34 @@ def dr_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: Optional[torc
              _ptr(cu_seqlens), _ptr(slots), B, H, G, d, e, int(gb is not None), int(bool(silu)), _stream()), "dr_scan")
 
 
+def dr_scan_pieces(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+                   slots: torch.Tensor, piece_cu: torch.Tensor, piece_slots: torch.Tensor, piece_state: torch.Tensor, B: int,
+                   pieces: int, H: int, d: int, e: int, silu: bool = False) -> None:
+    """`dr_scan` with one decay a head over a step of long prompts with every sequence cut into `pieces` pieces that are
+    walked side by side (twice: from a zero state, then from their true first states).  `piece_cu` int32 [B*pieces + 1]
+    cuts the packed tokens, `piece_slots` int32 [B*pieces] numbers the pieces (-1: a padding sequence's); `piece_state`
+    float [B*pieces, *glr_state_shape] is scratch."""
+    _dev("dr_scan_pieces", decay, out, slots, piece_cu, piece_slots, piece_state)
+    T = out.shape[0]
+    shape = tuple(glr_state_shape(H, d, e))
+    for name, t, w in (("q", q, H * d), ("k", k, H * d), ("v", v, H * e)):
+        _req(t.is_cuda and t.dtype == torch.float32 and t.shape == (T, w) and t.stride(1) == 1, f"dr_scan_pieces: {name} float32 [T, {w}]")
+    _req(T <= 1 or q.stride(0) == k.stride(0), "dr_scan_pieces: q and k rows equally far apart")
+    _req(decay.dtype == torch.float32 and decay.numel() == H, "dr_scan_pieces: decay float32 [H]")
+    _req(out.dtype == torch.float32 and out.shape == (T, H * e), "dr_scan_pieces: out float32 [T, H e]")
+    _req(state.is_cuda and state.dtype == torch.float32 and tuple(state.shape[1:]) == shape and state[0].is_contiguous(),
+         "dr_scan_pieces: state float32 [slots, *glr_state_shape], every slot's dense")
+    _req(piece_state.dtype == torch.float32 and piece_state.shape == (B * pieces,) + shape and piece_state.is_contiguous(),
+         "dr_scan_pieces: scratch of the wrong size")
+    _req(piece_cu.dtype == piece_slots.dtype == torch.int32 and piece_cu.numel() == B * pieces + 1 and piece_slots.numel() == B * pieces
+         and slots.numel() >= B, "dr_scan_pieces: piece arrays int32 [B*pieces + 1] and [B*pieces]")
+    qs = q.stride(0) if T > 1 else H * d
+    vs = v.stride(0) if T > 1 else H * e
+    f = _fn("delta_rule", "br_dr_scan_pieces", [_P, _P, c_size_t, _P, c_size_t, _P, _P, _P, c_size_t, _P, _P, _P, _P] + [c_int] * 6 + [_P])
+    _check(f(_ptr(q), _ptr(k), qs, _ptr(v), vs, _ptr(decay), _ptr(out), _ptr(state), state.stride(0), _ptr(slots), _ptr(piece_cu),
+             _ptr(piece_slots), _ptr(piece_state), B, pieces, H, d, e, int(bool(silu)), _stream()), "dr_scan_pieces")
+
+
 def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
     _dev("tanh", x, out)
     _req(x.dtype == torch.float32 and x.numel() == out.numel(), "tanh: x float32, out of the same size")

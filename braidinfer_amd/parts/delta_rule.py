@@ -33,6 +33,7 @@ from ..cache import StateNeed
 from ..errors import ConfigError, StepError
 from ..weights import TensorSpec
 from .base import Mixer, MixerContext, Runtime, register_part
+from .gated_recurrence import HGRN2, pieces_for
 from .linear import fused_layout, linear, stream_layout
 
 
@@ -123,6 +124,7 @@ class LightningAttention(Mixer):
     through_linear_only = True
 
     NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "norm": "norm", "o": "o"}
+    MIN_PIECE = 128          # tokens: shorter pieces do not pay for the second walk
 
     def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, decay: Sequence[float], norm_eps: float,
                  out_scale: float = 1.0, names: Optional[Dict[str, str]] = None):
@@ -165,8 +167,17 @@ class LightningAttention(Mixer):
         rows = step.ws.get("la_rows", (T, 2 * hd + 2 * he), torch.float32)
         linear(h, self.w_in, rows, step.ws)
         o = step.ws.get("la_o", (T, he), torch.float32)
-        K.dr_scan(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], None, self.decay, o, ctx.state,
-                  step.cu_seqlens, step.slots, step.n_seqs, nh, nh, d, e, silu=True)
+        pieces = pieces_for(step, nh * -(-e // 16), self.MIN_PIECE)
+        if pieces > 1:
+            # long prompts: the recurrence is linear in the state, so every sequence is cut into pieces that are walked
+            # side by side, twice
+            cu, numbers = HGRN2._piece_arrays(step, pieces)
+            piece_state = step.ws.get("la_piece_state", (step.n_seqs * pieces,) + tuple(K.glr_state_shape(nh, d, e)), torch.float32)
+            K.dr_scan_pieces(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], self.decay, o, ctx.state, step.slots,
+                             cu, numbers, piece_state, step.n_seqs, pieces, nh, d, e, silu=True)
+        else:
+            K.dr_scan(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], None, self.decay, o, ctx.state,
+                      step.cu_seqlens, step.slots, step.n_seqs, nh, nh, d, e, silu=True)
         y = step.ws.get("la_y", (T, he), self.rt.dtype)
         # all heads normed together: one "head" of H e channels
         K.head_norm_gate(o, self.norm_w, rows[:, 2 * hd + he:], y, 1, he, self.eps, gate_sigmoid=True)

@@ -353,6 +353,56 @@ def test_decayed_outer_sum_scan(H, d, e):
             assert np.abs(dense[i][h] - S).max() < 3e-5 * max(1.0, np.abs(S).max())
 
 
+@pytest.mark.parametrize("H,d,e,pieces", [(3, 16, 24, 3), (1, 80, 72, 5), (2, 128, 128, 4), (2, 9, 5, 2)])
+def test_decayed_outer_sum_in_pieces(H, d, e, pieces):
+    """Long portions cut into pieces that are walked side by side: two sequences with states left by an earlier portion,
+    a padding sequence between them, pieces of unequal length and an empty one."""
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(H + d + pieces)
+    lens, first = [150, 61], [30, 5]
+    decay = np.array([1.0, 0.0, 0.9][:H] if H > 1 else [0.97], dtype=np.float32)
+    q, k, v = ([f32(rng.standard_normal((n, H * w))) for n in lens] for w in (d, d, e))
+    shape = tuple(K.glr_state_shape(H, d, e))
+    state = torch.zeros((6,) + shape, dtype=torch.float32, device="cuda")
+    slots_of = [4, 1]
+    got = [[], []]
+    # the first portions by the plain walk
+    new = [first[0], 1, first[1]]
+    cat = lambda seqs, lo, n, width: torch.tensor(np.concatenate([seqs[0][lo[0]:lo[0] + n[0]], np.ones((1, width)),
+                                                                   seqs[1][lo[1]:lo[1] + n[1]]]).astype(np.float32)).cuda()
+    o = torch.zeros((sum(new), H * e), dtype=torch.float32, device="cuda")
+    K.dr_scan(cat(q, [0, 0], first, H * d), cat(k, [0, 0], first, H * d), cat(v, [0, 0], first, H * e), None, dev_f(decay), o, state,
+              dev_i(np.cumsum([0] + new)), dev_i([slots_of[0], -1, slots_of[1]]), 3, H, H, d, e, silu=True)
+    got[0].append(o.cpu().numpy()[:first[0]])
+    got[1].append(o.cpu().numpy()[first[0] + 1:])
+    # the rest in pieces: runs of equal length, the last ones shorter or empty
+    rest = [lens[0] - first[0], lens[1] - first[1]]
+    new = [rest[0], 1, rest[1]]
+    cu, numbers, at = [0], [], 0
+    for b, n in enumerate(new):
+        run = -(-(-(-n // pieces)) // 16) * 16
+        for c in range(pieces):
+            cu.append(at + min(n, (c + 1) * run))
+            numbers.append(b * pieces + c if b != 1 else -1)
+        at += n
+    assert any(cu[i] == cu[i + 1] for i in range(len(cu) - 1))
+    o = torch.full((sum(new), H * e), 7.0, dtype=torch.float32, device="cuda")
+    scratch = torch.full((3 * pieces,) + shape, 5.0, dtype=torch.float32, device="cuda")
+    K.dr_scan_pieces(cat(q, first, rest, H * d), cat(k, first, rest, H * d), cat(v, first, rest, H * e), dev_f(decay), o, state,
+                     dev_i([slots_of[0], -1, slots_of[1]]), dev_i(cu), dev_i(numbers), scratch, 3, pieces, H, d, e, silu=True)
+    got[0].append(o.cpu().numpy()[:rest[0]])
+    got[1].append(o.cpu().numpy()[rest[0] + 1:])
+    for i in range(2):
+        g_ = np.concatenate(got[i])
+        for h in range(H):
+            want, S = P.decayed_outer_sum(P.silu(q[i][:, h * d:(h + 1) * d]), P.silu(k[i][:, h * d:(h + 1) * d]), P.silu(v[i][:, h * e:(h + 1) * e]),
+                                          float(decay[h]), return_state=True)
+            assert np.abs(g_[:, h * e:(h + 1) * e] - want).max() < 3e-5 * max(1.0, np.abs(want).max()), f"sequence {i} head {h}"
+            dense = K.glr_state_dense(state[slots_of[i]], H, d, e).cpu().numpy()[h]
+            assert np.abs(dense - S).max() < 3e-5 * max(1.0, np.abs(S).max())
+    assert float(state[[0, 2, 3, 5]].abs().max()) == 0
+
+
 def test_order_of_decay_correction_write_and_read():
     """Inputs that tell the order apart: the read-out sees the token's own write; the decay comes before the correction;
     a repeated key with full write strength replaces what lay under it; no write strength leaves the state alone."""
@@ -380,7 +430,7 @@ def test_head_norms_with_both_gates():
     gate; the gates read from inside wider rows."""
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(4)
-    for T, H, e in ((7, 3, 33), (2, 1, 80), (5, 4, 16), (1, 6, 7)):
+    for T, H, e in ((7, 3, 33), (2, 1, 80), (5, 4, 16), (1, 6, 7), (3, 8, 128), (2, 2, 600)):       # rows of 512 channels and more take a workgroup each
         o = rng.standard_normal((T, H * e)).astype(np.float32) * 3
         o[0] *= 1e-3                                            # a row so small that eps inside the root matters
         w1 = (1 + 0.3 * rng.standard_normal(e)).astype(np.float32)
