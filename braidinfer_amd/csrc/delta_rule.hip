@@ -95,6 +95,84 @@ __global__ __launch_bounds__(256) void dr_conv_prepare_kernel(
     }
 }
 
+// The same with four channels a lane through 16-byte loads, for widths that are multiples of 4 (d, e, `width`, the kept
+// rows' stride; 16-byte aligned pointers): `taps_t` [n, C] holds the taps with the channels side by side.  LPH lanes a
+// (token, head row), 64 / LPH of them a wave: 16 lanes for heads of up to 64 channels, 32 up to 128, else 64.
+template <int LPH>
+__global__ __launch_bounds__(256) void dr_conv_prepare_vec_kernel(
+    const float* __restrict__ rows, int width, const float* __restrict__ taps_t, int n_taps,
+    const float* __restrict__ kept, size_t kept_stride, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, float* __restrict__ qo, float* __restrict__ ko, float* __restrict__ vo,
+    float* __restrict__ gb, int T, int G, int H, int d, int e) {
+    constexpr int NJ = LPH == 64 ? DR_MAX_EPL / 4 : 1;
+    const int n_hr = 2 * G + H;
+    const int lane = threadIdx.x & 63, l = lane % LPH;
+    const long long unit = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / LPH) + lane / LPH;
+    const bool on = unit < (long long)T * n_hr;          // lanes behind the last row go along for the sums and write nothing
+    const int t = on ? (int)(unit / n_hr) : 0, hr = on ? (int)(unit - (long long)t * n_hr) : 0;
+    const bool is_q = hr < G, is_k = !is_q && hr < 2 * G;
+    const int head = is_q ? hr : (is_k ? hr - G : hr - 2 * G);
+    const int n = (is_q || is_k) ? d : e;
+    const int C = 2 * G * d + H * e;
+    const int col0 = is_q ? head * d : (is_k ? G * d + head * d : 2 * G * d + head * e);
+    const int b = seq_of_token[t];
+    const int slot = slots[b], t0 = cu_seqlens[b];
+    const int i_in_step = t - t0;
+    f32x4 v[NJ];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int i = 4 * l + 4 * LPH * j;
+        v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (on && i < n) {
+            const int ch = col0 + i;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int x = 0; x < n_taps; ++x) {
+                const int ii = i_in_step - (n_taps - 1) + x;          // the input's place in the step
+                f32x4 in = {0.f, 0.f, 0.f, 0.f};
+                if (ii >= 0) in = *(const f32x4*)(rows + (size_t)(t0 + ii) * width + ch);
+                else if (slot >= 0) in = *(const f32x4*)(kept + (size_t)slot * kept_stride + (size_t)(n_taps - 1 + ii) * C + ch);
+                const f32x4 w = *(const f32x4*)(taps_t + (size_t)x * C + ch);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[c] = fmaf(w[c], in[c], acc[c]);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                v[j][c] = dr_silu(acc[c]);
+                ss = fmaf(v[j][c], v[j][c], ss);
+            }
+        }
+    }
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);          // over the row's lanes, in a fixed order
+    if (!on) return;
+    float mult = 1.f;
+    if (is_q || is_k) {
+        mult = 1.0f / sqrtf(ss + 1e-6f);
+        if (is_q) mult *= 1.0f / sqrtf((float)d);
+    }
+    float* dst = is_q ? qo + (size_t)t * G * d + head * d : (is_k ? ko + (size_t)t * G * d + head * d
+                                                                   : vo + (size_t)t * H * e + head * e);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int i = 4 * l + 4 * LPH * j;
+        if (i < n) {
+            f32x4 out;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) out[c] = v[j][c] * mult;
+            *(f32x4*)(dst + i) = out;
+        }
+    }
+    if (!is_q && !is_k && l == 0) {
+        const float braw = rows[(size_t)t * width + C + head];
+        const float araw = rows[(size_t)t * width + C + H + head] + dt_bias[head];
+        const float sp = araw > 20.f ? araw : log1pf(expf(araw));
+        gb[(size_t)t * 2 * H + head] = expf(-expf(a_log[head]) * sp);
+        gb[(size_t)t * 2 * H + H + head] = 1.0f / (1.0f + expf(-braw));
+    }
+}
+
 // After the step: every sequence's last n - 1 inputs into its slot.  grid (B, ceil(C / 256)).
 __global__ __launch_bounds__(256) void dr_conv_keep_kernel(const float* __restrict__ rows, int width, int n_taps,
                                                            float* __restrict__ kept, size_t kept_stride,
@@ -113,7 +191,7 @@ __global__ __launch_bounds__(256) void dr_conv_keep_kernel(const float* __restri
     }
 }
 
-extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* taps, int n_taps, float* kept,
+extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* taps, const float* taps_t, int n_taps, float* kept,
                                   size_t kept_stride, const float* a_log, const float* dt_bias, const int* seq_of_token,
                                   const int* cu_seqlens, const int* slots, float* qo, float* ko, float* vo, float* gb,
                                   int T, int B, int G, int H, int d, int e, hipStream_t s) {
@@ -125,7 +203,18 @@ extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* tap
         (n_taps > 1 && (!kept || kept_stride < (size_t)(n_taps - 1) * C)) || !a_log || !dt_bias)
         return BR_BAD_ARG;
     const unsigned blocks = (unsigned)(((long long)T * (2 * G + H) + 3) / 4);
-    dr_conv_prepare_kernel<<<blocks, 256, 0, s>>>(rows, width, taps, n_taps, kept, kept_stride, a_log, dt_bias, seq_of_token,
+    auto at16 = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool vec = taps_t && d % 4 == 0 && e % 4 == 0 && width % 4 == 0 && at16(rows) && at16(taps_t) && at16(qo) && at16(ko) &&
+                     at16(vo) && (n_taps == 1 || (kept_stride % 4 == 0 && at16(kept)));
+    if (vec) {
+        const int widest = d > e ? d : e, lph = widest <= 64 ? 16 : (widest <= 128 ? 32 : 64);
+        const unsigned vblocks = (unsigned)(((long long)T * (2 * G + H) + 4 * (64 / lph) - 1) / (4 * (64 / lph)));
+#define DR_PREP(L) dr_conv_prepare_vec_kernel<L><<<vblocks, 256, 0, s>>>(rows, width, taps_t, n_taps, kept, kept_stride, a_log, dt_bias, \
+                                                                        seq_of_token, cu_seqlens, slots, qo, ko, vo, gb, T, G, H, d, e)
+        if (lph == 16) DR_PREP(16); else if (lph == 32) DR_PREP(32); else DR_PREP(64);
+#undef DR_PREP
+    }
+    else dr_conv_prepare_kernel<<<blocks, 256, 0, s>>>(rows, width, taps, n_taps, kept, kept_stride, a_log, dt_bias, seq_of_token,
                                                  cu_seqlens, slots, qo, ko, vo, gb, T, G, H, d, e);
     int rc = br_check_launch();
     if (rc != BR_OK || n_taps == 1) return rc;

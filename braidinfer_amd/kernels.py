@@ -862,13 +862,14 @@ def head_norm_gate(o: torch.Tensor, w: Optional[torch.Tensor], gate: Optional[to
 def dr_conv_prepare(rows: torch.Tensor, taps: torch.Tensor, kept: Optional[torch.Tensor], a_log: torch.Tensor,
                     dt_bias: torch.Tensor, seq_of_token: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor,
                     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: torch.Tensor, B: int, G: int, H: int, d: int,
-                    e: int) -> None:
+                    e: int, taps_t: Optional[torch.Tensor] = None) -> None:
     """rows float [T, >= C + 2 H] with C = 2 G d + H e: the sums q | k | v | b | a of a gated delta rule's projections.
     The first C columns pass a causal convolution over time per channel (taps float [C, n], the last column the current
     token's; `kept` a float view [slots, (n - 1) * C] of every sequence's last inputs, read and then brought up to
     date) and silu; q and k become unit vectors per head (q times d^-1/2); gb [T, 2 H] takes
-    g = exp(-exp(a_log) softplus(a + dt_bias)) and beta = sigmoid(b)."""
-    _dev("dr_conv_prepare", rows, taps, a_log, dt_bias, seq_of_token, cu_seqlens, slots, q, k, v, gb)
+    g = exp(-exp(a_log) softplus(a + dt_bias)) and beta = sigmoid(b).  `taps_t` float [n, C], the same taps with the channels
+    side by side, lets widths that are multiples of 4 go four channels a lane."""
+    _dev("dr_conv_prepare", rows, taps, a_log, dt_bias, seq_of_token, cu_seqlens, slots, q, k, v, gb, taps_t)
     T = rows.shape[0]
     C = 2 * G * d + H * e
     n = taps.shape[1] if taps.dim() == 2 else 0
@@ -883,8 +884,9 @@ def dr_conv_prepare(rows: torch.Tensor, taps: torch.Tensor, kept: Optional[torch
         _req(kept is not None and kept.is_cuda and kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] == (n - 1) * C
              and kept.stride(1) == 1, "dr_conv_prepare: kept float32 [slots, (n - 1) * C]")
         ks = kept.stride(0)
-    f = _fn("delta_rule", "br_dr_conv_prepare", [_P, c_int, _P, c_int, _P, c_size_t, _P, _P, _P, _P, _P, _P, _P, _P, _P] + [c_int] * 6 + [_P])
-    _check(f(_ptr(rows), int(rows.shape[1]), _ptr(taps), n, _ptr(kept) if n > 1 else c_void_p(0), ks, _ptr(a_log), _ptr(dt_bias),
+    _req(taps_t is None or (taps_t.dtype == torch.float32 and taps_t.shape == (n, C) and taps_t.is_contiguous()), "dr_conv_prepare: taps_t float32 [n, C]")
+    f = _fn("delta_rule", "br_dr_conv_prepare", [_P, c_int, _P, _P, c_int, _P, c_size_t, _P, _P, _P, _P, _P, _P, _P, _P, _P] + [c_int] * 6 + [_P])
+    _check(f(_ptr(rows), int(rows.shape[1]), _ptr(taps), _ptr(taps_t), n, _ptr(kept) if n > 1 else c_void_p(0), ks, _ptr(a_log), _ptr(dt_bias),
              _ptr(seq_of_token), _ptr(cu_seqlens), _ptr(slots), _ptr(q), _ptr(k), _ptr(v), _ptr(gb), T, B, G, H, d, e, _stream()),
            "dr_conv_prepare")
 

@@ -63,7 +63,7 @@ class GatedDeltaRule(Mixer):
         self.names = dict(self.NAMES, **(names or {}))
         self.C = 2 * self.ng * self.d + self.nh * self.e          # convolved channels: q | k | v
         self.state_floats = _floats(K.glr_state_shape(self.nh, self.d, self.e))
-        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm_w = None
+        self.w_in = self.w_o = self.conv = self.conv_t = self.a_log = self.dt_bias = self.norm_w = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         n, gd, he = self.names, self.ng * self.d, self.nh * self.e
@@ -89,6 +89,7 @@ class GatedDeltaRule(Mixer):
         self.w_o = stream_layout(tensors[prefix + n["o"]], rt)
         self.conv = rt.own(torch.cat([tensors[prefix + n[x]].to(torch.float32).reshape(-1, self.taps)
                                       for x in ("q_conv", "k_conv", "v_conv")]))
+        self.conv_t = rt.own(self.conv.t().contiguous())          # [taps, channels]: four channels a lane where the widths allow
         self.a_log = rt.own(tensors[prefix + n["A_log"]].to(torch.float32).reshape(-1))
         self.dt_bias = rt.own(tensors[prefix + n["dt_bias"]].to(torch.float32).reshape(-1))
         # the head norm's weight for every head, with the mixer's multiplier
@@ -110,7 +111,7 @@ class GatedDeltaRule(Mixer):
         gb = step.ws.get("dr_gb", (T, 2 * nh), torch.float32)
         kept = ctx.state[:, self.state_floats:] if self.taps > 1 else None
         K.dr_conv_prepare(rows, self.conv, kept, self.a_log, self.dt_bias, step.seq_of_token, step.cu_seqlens, step.slots,
-                          q, k, v, gb, step.n_seqs, ng, nh, d, e)
+                          q, k, v, gb, step.n_seqs, ng, nh, d, e, taps_t=self.conv_t)
         o = step.ws.get("dr_o", (T, nh * e), torch.float32)
         S = ctx.state[:, :self.state_floats].view((-1,) + tuple(K.glr_state_shape(nh, d, e)))
         K.dr_scan(q, k, v, gb, None, o, S, step.cu_seqlens, step.slots, step.n_seqs, nh, ng, d, e)

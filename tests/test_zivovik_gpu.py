@@ -233,14 +233,16 @@ def test_norm_weights_around_zero_and_a_normed_branch_added():
     assert np.abs(acc.cpu().numpy() - (acc0 + 0.35 * P.plain_norm(f32(x), stored + 1.0, eps))).max() < 1e-6
 
 
-@pytest.mark.parametrize("G,H,d,e,taps", [(2, 4, 6, 10, 3), (1, 1, 80, 72, 1), (2, 2, 16, 24, 4), (3, 6, 33, 7, 2), (1, 2, 130, 8, 16)])
-def test_convolution_unit_vectors_decay_and_write_strength(G, H, d, e, taps):
+@pytest.mark.parametrize("G,H,d,e,taps,by_four", [(2, 4, 6, 10, 3, False), (1, 1, 80, 72, 1, False), (2, 2, 16, 24, 4, False), (3, 6, 33, 7, 2, False),
+                                                 (1, 2, 130, 8, 16, False), (2, 2, 16, 24, 4, True), (1, 1, 80, 72, 1, True), (2, 4, 128, 128, 4, True),
+                                                 (1, 2, 300, 260, 3, True)])
+def test_convolution_unit_vectors_decay_and_write_strength(G, H, d, e, taps, by_four):
     """The step in front of the delta rule: two sequences in unequal portions down to single tokens, the last inputs
     kept in slots that are not neighbours and lie inside wider rows, a padding sequence between them."""
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(G * 100 + taps)
     C = 2 * G * d + H * e
-    width = C + 2 * H + 5                        # the projection's rows carry further columns behind
+    width = C + 2 * H + (4 - (C + 2 * H) % 4 if by_four else 5)       # the projection's rows carry further columns behind
     lens = [41, 9]
     raw = [rng.standard_normal((n, width)).astype(np.float32) * 1.5 for n in lens]
     w_taps = (rng.standard_normal((C, taps)) * 0.6).astype(np.float32)
@@ -255,8 +257,9 @@ def test_convolution_unit_vectors_decay_and_write_strength(G, H, d, e, taps):
         g = np.exp(-np.exp(f32(a_log)) * P.softplus(r[:, C + H:C + 2 * H] + f32(dt_bias)))
         want.append((q.reshape(-1, G * d), k.reshape(-1, G * d), c[:, 2 * G * d:], np.concatenate([g, beta], axis=1)))
     n_kept = (taps - 1) * C
-    arena = torch.zeros((6, n_kept + 9), dtype=torch.float32, device="cuda")
+    arena = torch.zeros((6, n_kept + (8 if by_four else 9)), dtype=torch.float32, device="cuda")
     kept = arena[:, 4:4 + n_kept] if taps > 1 else None
+    taps_t = dev_f(np.ascontiguousarray(w_taps.T)) if by_four else None          # four channels a lane through 16-byte loads
     slots_of = [4, 1]
     got = [[[] for _ in range(4)] for _ in lens]
     at = [0, 0]
@@ -268,7 +271,7 @@ def test_convolution_unit_vectors_decay_and_write_strength(G, H, d, e, taps):
         q, k = torch.zeros((T, G * d), device="cuda"), torch.zeros((T, G * d), device="cuda")
         v, gb = torch.zeros((T, H * e), device="cuda"), torch.zeros((T, 2 * H), device="cuda")
         K.dr_conv_prepare(rows, dev_f(w_taps), kept, dev_f(a_log), dev_f(dt_bias), dev_i(np.repeat(np.arange(3), new)),
-                          dev_i(np.cumsum([0] + new)), dev_i([slots_of[0], -1, slots_of[1]]), q, k, v, gb, 3, G, H, d, e)
+                          dev_i(np.cumsum([0] + new)), dev_i([slots_of[0], -1, slots_of[1]]), q, k, v, gb, 3, G, H, d, e, taps_t=taps_t)
         for i, lo in ((0, 0), (1, portion[0] + 1)):
             for j, t in enumerate((q, k, v, gb)):
                 got[i][j].append(t.cpu().numpy()[lo:lo + portion[i]])
