@@ -75,7 +75,7 @@ LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_
              "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax", "wkv_scan", "wkv_scan_pieces", "shift_mix", "head_norm_gate", "tanh",
              "latent_prepare", "head_linear", "route_topk", "experts_up", "experts_down", "experts_sort", "experts_gather",
              "experts_combine", "experts_up_grouped", "experts_down_grouped", "experts_gemm", "clamped_glu", "add_bias_rows",
-             "add_position_rows", "pwa_gate", "dr_conv_prepare", "dr_scan", "dr_scan_pieces"]
+             "add_position_rows", "pwa_gate", "dr_conv_prepare", "dr_scan", "dr_scan_pieces", "silu_rows"]
 
 
 def kernel_share(torch, eng, entries_of, classes):

@@ -223,6 +223,38 @@ extern "C" int br_dr_conv_prepare(const float* rows, int width, const float* tap
     return br_check_launch();
 }
 
+// x[t, :n] <- silu(x[t, :n]) in place on float rows `stride` apart (projections' sums that go on as activations: done
+// once here, not by every workgroup of a scan that reads them).  VEC: four a thread, for n, stride and pointer in fours.
+template <bool VEC>
+__global__ __launch_bounds__(256) void dr_silu_rows_kernel(float* __restrict__ x, size_t stride, int n, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    if (VEC) {
+        const size_t per = (size_t)n / 4, t = i / per, c = (i - t * per) * 4;
+        f32x4* p = (f32x4*)(x + t * stride + c);
+        f32x4 v = *p;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = dr_silu(v[k]);
+        *p = v;
+    } else {
+        const size_t t = i / n, c = i - t * n;
+        float* p = x + t * stride + c;
+        *p = dr_silu(*p);
+    }
+}
+
+extern "C" int br_silu_rows(float* x, size_t stride, int T, int n, hipStream_t s) {
+    if (T <= 0 || n <= 0) return BR_OK;
+    if (stride < (size_t)n) return BR_BAD_ARG;
+    const bool vec = n % 4 == 0 && stride % 4 == 0 && ((uintptr_t)x % 16) == 0;
+    const size_t total = vec ? (size_t)T * (n / 4) : (size_t)T * n;
+    const size_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffULL) return BR_BAD_ARG;
+    if (vec) dr_silu_rows_kernel<true><<<(unsigned)blocks, 256, 0, s>>>(x, stride, n, total);
+    else dr_silu_rows_kernel<false><<<(unsigned)blocks, 256, 0, s>>>(x, stride, n, total);
+    return br_check_launch();
+}
+
 // ---------------------------------------------------------------------- scan -------
 // q, k: float rows `qk_stride` apart, head kh's d channels at kh * d (kh = h / (H / G): G heads of keys serve H
 // heads of values); v: rows `v_stride` apart, head h's e channels at h * e.  DELTA: g and beta per token and

@@ -919,6 +919,14 @@ def dr_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: Optional[torc
              _ptr(cu_seqlens), _ptr(slots), B, H, G, d, e, int(gb is not None), int(bool(silu)), _stream()), "dr_scan")
 
 
+def silu_rows(x: torch.Tensor) -> None:
+    """x <- silu(x) in place: a float view [T, n] whose rows may be strided (some columns of a projection's sums)."""
+    _req(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "silu_rows: a float32 view [T, n] with dense rows")
+    T, n = x.shape
+    f = _fn("delta_rule", "br_silu_rows", [_P, c_size_t, c_int, c_int, _P])
+    _check(f(_ptr(x), x.stride(0) if T > 1 else n, T, n, _stream()), "silu_rows")
+
+
 def dr_scan_pieces(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
                    slots: torch.Tensor, piece_cu: torch.Tensor, piece_slots: torch.Tensor, piece_state: torch.Tensor, B: int,
                    pieces: int, H: int, d: int, e: int, silu: bool = False) -> None:

@@ -174,8 +174,10 @@ class LightningAttention(Mixer):
             # side by side, twice
             cu, numbers = HGRN2._piece_arrays(step, pieces)
             piece_state = step.ws.get("la_piece_state", (step.n_seqs * pieces,) + tuple(K.glr_state_shape(nh, d, e)), torch.float32)
+            # two walks by many workgroups a head: the activation once, ahead of them
+            K.silu_rows(rows[:, :2 * hd + he])
             K.dr_scan_pieces(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], self.decay, o, ctx.state, step.slots,
-                             cu, numbers, piece_state, step.n_seqs, pieces, nh, d, e, silu=True)
+                             cu, numbers, piece_state, step.n_seqs, pieces, nh, d, e, silu=False)
         else:
             K.dr_scan(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], None, self.decay, o, ctx.state,
                       step.cu_seqlens, step.slots, step.n_seqs, nh, nh, d, e, silu=True)

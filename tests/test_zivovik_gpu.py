@@ -406,6 +406,19 @@ def test_decayed_outer_sum_in_pieces(H, d, e, pieces):
     assert float(state[[0, 2, 3, 5]].abs().max()) == 0
 
 
+def test_silu_of_some_columns_in_place():
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(11)
+    for T, width, lo, n in ((9, 40, 0, 24), (5, 37, 3, 30), (1, 16, 4, 8), (300, 64, 8, 52)):
+        x0 = (rng.standard_normal((T, width)) * 4).astype(np.float32)
+        x = dev_f(x0)
+        K.silu_rows(x[:, lo:lo + n])
+        want = f32(x0).copy()
+        want[:, lo:lo + n] = P.silu(want[:, lo:lo + n])
+        assert np.abs(x.cpu().numpy() - want).max() < 1e-6 * np.abs(want).max()
+        assert np.array_equal(x.cpu().numpy()[:, :lo], x0[:, :lo]) and np.array_equal(x.cpu().numpy()[:, lo + n:], x0[:, lo + n:])
+
+
 def test_order_of_decay_correction_write_and_read():
     """Inputs that tell the order apart: the read-out sees the token's own write; the decay comes before the correction;
     a repeated key with full write strength replaces what lay under it; no write strength leaves the state alone."""
