@@ -805,6 +805,27 @@ def test_greedy_generation_through_the_engine(folders, engines):
                 break
 
 
+def test_the_command_line_generates_from_a_zivovik_folder(folders):
+    """`bin/generate` on a Zivovik folder: the model class by config.json, greedy tokens as the plain implementation's;
+    a sampled run ends and stays inside the vocabulary."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, cfg, w = folders[("a", "float32")]
+    p = [7, 3, 200, 5, 11]
+    want = P.greedy_generate(cfg, w, p, 6)
+    env = dict(os.environ, MODEL=folder, MAX_TOKENS="6")
+    gen = [sys.executable, os.path.join(root, "bin", "generate"), "--dtype", "float32", "--prompt-ids", ",".join(map(str, p))]
+    r = subprocess.run(gen, env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    assert [int(t) for t in r.stdout.split()] == want
+    r = subprocess.run(gen + ["--temperature", "0.8", "--top-k", "20", "--seed", "5"], env=env, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    toks = [int(t) for t in r.stdout.split()]
+    assert len(toks) == 6 and all(0 <= t < cfg["vocab"] for t in toks)
+
+
 def test_presets_run(tmp_path):
     """The tiny preset as a random-weights folder of the library's own making, against the plain implementation."""
     import braidinfer_amd as B
