@@ -267,8 +267,8 @@ def _with(layer, mlp):
 
 
 # Shapes without a model folder: a tiny one for tests and tools, and two of the size of a real model's layers (eight
-# layer runs each: an attention layer, a parallel and a lightning layer passed three times, a closing attention layer;
-# a token's share of the experts equals a dense layer's inner width of 5,632 / 14,336).
+# layer runs each: a parallel and a lightning layer passed three times, then two attention layers; a token's share of
+# the experts equals a dense layer's inner width of 5,632 / 14,336).
 PRESETS: Dict[str, Dict[str, Any]] = {
     "zivovik-tiny": dict(vocab=320, width=96, max_positions=512, norm={"eps": 1e-5}, embedding={"scale": 2.0}, residual_mult=0.7,
                          loop={"start": 1, "stop": 3, "times": 2}, layers=[
@@ -276,17 +276,17 @@ PRESETS: Dict[str, Dict[str, Any]] = {
         _with(_parallel(3, 1, 16, 24, 4, 2, 16, 24, conv=4, every=8), _moe(48, 6, 2)),
         _with(_lightning(3, 16, 24), None),
         _with(_attention(4, 2, 24, every=16), _moe(48, 6, 2))]),
-    "zivovik-1b": dict(vocab=32768, width=2048, max_positions=16384, norm={"eps": 1e-6}, embedding={"scale": 1.0}, residual_mult=0.5,
-                       loop={"start": 1, "stop": 3, "times": 3}, layers=[
-        _with(_attention(16, 4, 128), _moe(1408, 16, 4)),
+    "zivovik-1b": dict(vocab=32768, width=2048, max_positions=16384, norm={"eps": 1e-6}, embedding={"scale": 1.0}, residual_mult=0.6,
+                       loop={"start": 0, "stop": 2, "times": 3}, layers=[
         _with(_parallel(8, 4, 128, 128, 16, 8, 128, 128), _moe(1408, 16, 4)),
         _with(_lightning(16, 128, 128), _moe(1408, 16, 4)),
+        _with(_attention(16, 4, 128), _moe(1408, 16, 4)),
         _with(_attention(16, 4, 128), _moe(1408, 16, 4))]),
-    "zivovik-7b": dict(vocab=32768, width=4096, max_positions=16384, norm={"eps": 1e-6}, embedding={"scale": 1.0}, residual_mult=0.5,
-                       loop={"start": 1, "stop": 3, "times": 3}, layers=[
-        _with(_attention(32, 8, 128), _moe(1792, 32, 8)),
+    "zivovik-7b": dict(vocab=32768, width=4096, max_positions=16384, norm={"eps": 1e-6}, embedding={"scale": 1.0}, residual_mult=0.6,
+                       loop={"start": 0, "stop": 2, "times": 3}, layers=[
         _with(_parallel(16, 8, 128, 128, 32, 16, 128, 128), _moe(1792, 32, 8)),
         _with(_lightning(32, 128, 128), _moe(1792, 32, 8)),
+        _with(_attention(32, 8, 128), _moe(1792, 32, 8)),
         _with(_attention(32, 8, 128), _moe(1792, 32, 8))]),
 }
 

@@ -48,9 +48,9 @@ def model(width, vocab, layers, loop, eps=1e-5, emb=2.0, mult=0.7, positions=102
 
 
 CONFIGS = {
-    # the usual stack: attention, then a parallel and a lightning layer passed three times, a closing attention layer
+    # the usual stack: attention, then a parallel and a lightning layer passed four times, a closing attention layer
     "a": model(64, 211, [att(4, 2, 16, every=16, mlp=moe(32, 6, 2)), par((3, 1, 16, 24, 0.3, 24), (4, 2, 16, 24, 4), mlp=moe(32, 6, 2)),
-                         lig(3, 16, 24, (0.6, 0.9, 0.995), mlp=moe(32, 6, 2)), att(4, 2, 16, every=16, mlp=moe(32, 6, 2))], (1, 3, 3)),
+                         lig(3, 16, 24, (0.6, 0.9, 0.995), mlp=moe(32, 6, 2)), att(4, 2, 16, every=16, mlp=moe(32, 6, 2))], (1, 3, 4)),
     # sizes the usual shapes make equal or 1, and odd ones: the whole model passed twice, as many key heads as heads and
     # one head, head sizes that are no multiples of 4 or 8, a convolution of one tap (none) and of two, a decay of 1
     # (a plain sum) and a short memory, all experts chosen, one expert chosen, layers without feed-forward, an
@@ -742,8 +742,8 @@ def test_slots_and_pages_used_again(folders):
         want = P.forward(cfg, w, toks)
         close(run(eng, toks, [len(toks) - 10] + [1] * 10), want, "float32", f"request {r}")
     assert [g.pool.free_count for g in eng.cache.groups] == free_before
-    # a cache unit for every attention run and none for the lightning runs: runs 0 and 7, and the left sides at 1, 3, 5
-    assert sorted(eng.cache.group_of_unit) == [0, 1, 3, 5, 7]
+    # a cache unit for every attention run and none for the lightning runs: runs 0 and 9, and the left sides at 1, 3, 5, 7
+    assert sorted(eng.cache.group_of_unit) == [0, 1, 3, 5, 7, 9]
     # two requests side by side whose slots have just been used, one of them a single token long
     import braidinfer_amd as B
     a, b = tokens_of(cfg, 70, 90), tokens_of(cfg, 1, 91)
