@@ -68,11 +68,14 @@ CONFIGS = {
     # attention only, the first layer passed twice; every width equal, a scale of 1, two experts
     "e": model(32, 64, [att(2, 2, 16, coef=0.25, every=1, scale=1.0, mlp=moe(16, 2, 1)), att(2, 1, 16, coef=0.0, every=9, scale=1.0, mlp=moe(16, 2, 2))],
                (0, 1, 2)),
+    # sizes that the matrix-core attention kernels, the products' wide tiles and the grouped experts' kernels take
+    "f": model(256, 1000, [par((4, 2, 64, 128, 0.3, 32), (4, 2, 64, 128, 4), mlp=moe(128, 8, 2)), att(8, 2, 64, every=48, mlp=moe(128, 8, 2)),
+                           lig(4, 64, 64, (0.7, 0.9, 0.97, 0.999), mlp=moe(128, 8, 2))], (0, 2, 2)),
 }
 
 # The size of the random matrices: large enough for every layer to move the logits, small enough where a scale of 1
 # or a head of few channels would otherwise make a softmax so sharp that it amplifies bfloat16 rounding a hundredfold.
-GAINS = {"a": 1.3, "b": 1.0, "c": 1.3, "d": 1.3, "e": 0.7}
+GAINS = {"a": 1.3, "b": 1.0, "c": 1.3, "d": 1.3, "e": 0.7, "f": 1.0}
 
 
 # One expert chosen in front of a state that never forgets (a decay of 1) and a model passed twice: a single close call of
@@ -698,7 +701,7 @@ def test_portions_and_single_tokens(folders, engines, name, dtype):
             assert np.abs(got - whole).max() < 2e-4 * np.abs(whole).max()
 
 
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "f"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_unequal_batch_against_each_alone(folders, engines, name, dtype):
     import braidinfer_amd as B
@@ -754,7 +757,7 @@ def test_slots_and_pages_used_again(folders):
     close(lg, np.stack([P.forward(cfg, w, a)[69], P.forward(cfg, w, b)[0]]), "float32", "after the slots' earlier users")
 
 
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "f"])
 def test_long_decoding(folders, engines, name):
     """Three hundred single-token steps from a short prompt (recorded steps of the engine), past page borders and many
     steps of the temperature."""
