@@ -7,7 +7,7 @@ batched step function, a generation loop with the reference's sampler, and trace
 replay.  Every device operation is a hand-written HIP kernel under `csrc/`.
 """
 from .errors import BraidError, ConfigError, WeightError, CacheError, KernelError, StepError
-from .config import (MistralConfig, KesitarConfig, SidiraxConfig, ZivovikConfig, any_preset, preset, PRESETS, config_from_folder, config_from_dict, spec_of,
+from .config import (MistralConfig, KesitarConfig, SidiraxConfig, ZivovikConfig, LadadraConfig, any_preset, preset, PRESETS, config_from_folder, config_from_dict, spec_of,
                      register_architecture, registered_architectures, PartSpec, LayerSpec, ScheduleEntry,
                      ModelSpec, prenorm_layer)
 from .parts import register_part
@@ -17,7 +17,7 @@ from .sampling import SamplingParams, Sampler
 __version__ = "0.1.0"
 
 __all__ = ["BraidError", "ConfigError", "WeightError", "CacheError", "KernelError", "StepError",
-           "MistralConfig", "KesitarConfig", "SidiraxConfig", "ZivovikConfig", "any_preset", "preset", "PRESETS", "config_from_folder", "config_from_dict", "spec_of",
+           "MistralConfig", "KesitarConfig", "SidiraxConfig", "ZivovikConfig", "LadadraConfig", "any_preset", "preset", "PRESETS", "config_from_folder", "config_from_dict", "spec_of",
            "register_architecture", "registered_architectures", "PartSpec", "LayerSpec", "ScheduleEntry",
            "ModelSpec", "prenorm_layer", "register_part", "Engine", "StepEntry", "DecoderModel", "generate", "GenerationResult",
            "GenerationStats", "SamplingParams", "Sampler"]

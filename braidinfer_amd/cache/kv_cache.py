@@ -47,6 +47,9 @@ class CacheNeed:
     # values, say): a sequence of L tokens holds L // tokens_per_row rows, one for each complete block,
     # and pages are counted in rows.  Such a unit keeps all its rows (no window, no `live_from`).
     tokens_per_row: int = 1
+    # The first `keep_first` positions of a sequence stay readable whatever `window` or `live_from` say (a window that
+    # also keeps the sequence's first tokens): the pages that hold them are never returned.
+    keep_first: int = 0
 
     @property
     def key_dim(self) -> int:
@@ -122,7 +125,8 @@ class CacheGroup:
         self._staging = _PinnedStaging(max(4096, 2 * max_pages_per_seq)) if self.device.type == "cuda" else None
         if need.kv_heads <= 0 or need.key_dim <= 0 or need.val_dim < 0:
             raise CacheError(f"a cache unit needs kv heads and a key width above zero, got {need}")
-        if need.tokens_per_row < 1 or (need.tokens_per_row > 1 and (need.window is not None or need.live_from is not None)):
+        if need.tokens_per_row < 1 or need.keep_first < 0 or \
+                (need.tokens_per_row > 1 and (need.window is not None or need.live_from is not None or need.keep_first)):
             raise CacheError(f"a cache unit keeps one row for every tokens_per_row >= 1 tokens, and all of them when "
                              f"that is more than one, got {need}")
         self.key_elems = need.kv_heads * page_tokens * need.key_dim        # of one page
@@ -170,7 +174,8 @@ class CacheGroup:
         if self.need.window is None and self.need.live_from is None:
             return
         first_live = self.need.first_live(length) // self.page_tokens
-        lo = self.first_page[slot]
+        # pages that hold kept first tokens stay; `first_page` counts from behind them
+        lo = max(self.first_page[slot], -(-max(0, self.need.keep_first) // self.page_tokens))
         if first_live > lo:
             dead = [p for p in self.pages[slot][lo:first_live] if p >= 0]
             self.pool.free(dead)

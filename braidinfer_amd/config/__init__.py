@@ -6,7 +6,9 @@ from .mistral import MistralConfig, PRESETS, preset, build_spec as build_mistral
 from .kesitar import KesitarConfig, build_spec as build_kesitar_spec, ARCHITECTURE as KESITAR
 from .sidirax import SidiraxConfig, build_spec as build_sidirax_spec, ARCHITECTURE as SIDIRAX
 from .zivovik import ZivovikConfig, build_spec as build_zivovik_spec, ARCHITECTURE as ZIVOVIK
+from .ladadra import LadadraConfig, build_spec as build_ladadra_spec, ARCHITECTURE as LADADRA
 from . import kesitar as _kesitar
+from . import ladadra as _ladadra
 from . import zivovik as _zivovik
 from . import sidirax as _sidirax
 
@@ -14,8 +16,10 @@ register_architecture(MISTRAL, MistralConfig, build_mistral_spec, model_type="mi
 register_architecture(KESITAR, KesitarConfig, build_kesitar_spec, model_type="kesitar", replace=True)
 register_architecture(SIDIRAX, SidiraxConfig, build_sidirax_spec, model_type="sidirax", replace=True)
 register_architecture(ZIVOVIK, ZivovikConfig, build_zivovik_spec, model_type="zivovik", replace=True)
+register_architecture(LADADRA, LadadraConfig, build_ladadra_spec, model_type="ladadra", replace=True)
 PRESET_FAMILIES = {MISTRAL: (PRESETS, preset), KESITAR: (_kesitar.PRESETS, _kesitar.preset),
-                   SIDIRAX: (_sidirax.PRESETS, _sidirax.preset), ZIVOVIK: (_zivovik.PRESETS, _zivovik.preset)}
+                   SIDIRAX: (_sidirax.PRESETS, _sidirax.preset), ZIVOVIK: (_zivovik.PRESETS, _zivovik.preset),
+                   LADADRA: (_ladadra.PRESETS, _ladadra.preset)}
 
 
 def any_preset(name: str, **overrides):
@@ -31,5 +35,5 @@ __all__ = [
     "Architecture", "register_architecture", "unregister_architecture", "registered_architectures",
     "architecture_of", "architecture_of_config", "read_config_json", "config_from_dict",
     "config_from_folder", "spec_of", "generation_stop_tokens", "MistralConfig", "PRESETS", "preset",
-    "KesitarConfig", "SidiraxConfig", "ZivovikConfig", "any_preset", "PRESET_FAMILIES",
+    "KesitarConfig", "SidiraxConfig", "ZivovikConfig", "LadadraConfig", "any_preset", "PRESET_FAMILIES",
 ]

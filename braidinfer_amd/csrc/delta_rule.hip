@@ -255,6 +255,48 @@ extern "C" int br_silu_rows(float* x, size_t stride, int T, int n, hipStream_t s
     return br_check_launch();
 }
 
+// q and k rows (float sums of their projections, rows `stride` apart, `heads` heads of d channels each) turned in place
+// by their tokens' positions: of the first `rd` channels of a head, channel i < rd / 2 and channel i + rd / 2 form
+// a pair that is turned by the angle whose cosine and sine are cs[t, i], sn[t, i] ((u, v) -> (u c - v s, v c + u s));
+// the other channels pass.  Every channel of q is then multiplied by `q_mul` and every channel of k by `k_mul`.
+// A thread a channel below rd / 2 (it owns the pair) or from rd on; grid over T * heads * (d - rd / 2) threads.
+__global__ __launch_bounds__(256) void dr_rotate_rows_kernel(float* __restrict__ q, float* __restrict__ k, size_t stride,
+                                                             const float* __restrict__ cs, const float* __restrict__ sn,
+                                                             int rd, int heads, int d, float q_mul, float k_mul, size_t total) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int half = rd >> 1, per = d - half;
+    const size_t th = i / per;
+    const int j = (int)(i - th * per);
+    const size_t t = th / heads;
+    const int h = (int)(th - t * heads);
+    float* qr = q + t * stride + (size_t)h * d;
+    float* kr = k + t * stride + (size_t)h * d;
+    if (j < half) {
+        const float c = cs[t * half + j], s_ = sn[t * half + j];
+        const float qu = qr[j], qv = qr[j + half], ku = kr[j], kv = kr[j + half];
+        qr[j] = (qu * c - qv * s_) * q_mul;
+        qr[j + half] = (qv * c + qu * s_) * q_mul;
+        kr[j] = (ku * c - kv * s_) * k_mul;
+        kr[j + half] = (kv * c + ku * s_) * k_mul;
+    } else {
+        const int ch = j + half;                    // channels from rd on
+        qr[ch] *= q_mul;
+        kr[ch] *= k_mul;
+    }
+}
+
+extern "C" int br_dr_rotate_rows(float* q, float* k, size_t stride, const float* cs, const float* sn, int rd, int T, int heads,
+                                 int d, float q_mul, float k_mul, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (heads <= 0 || d <= 0 || rd < 0 || (rd & 1) || rd > d || stride < (size_t)heads * d || (rd > 0 && (!cs || !sn))) return BR_BAD_ARG;
+    const size_t total = (size_t)T * heads * (d - rd / 2);
+    const size_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffULL) return BR_BAD_ARG;
+    dr_rotate_rows_kernel<<<(unsigned)blocks, 256, 0, s>>>(q, k, stride, cs, sn, rd, heads, d, q_mul, k_mul, total);
+    return br_check_launch();
+}
+
 // ---------------------------------------------------------------------- scan -------
 // q, k: float rows `qk_stride` apart, head kh's d channels at kh * d (kh = h / (H / G): G heads of keys serve H
 // heads of values); v: rows `v_stride` apart, head h's e channels at h * e.  DELTA: g and beta per token and

@@ -184,7 +184,19 @@ __global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* _
             }
         }
     }
-    if (!ADD || !w2) return;
+    if (!ADD || !y2) return;
+    if (!w2) {      // no second norm: the new residual row as it is, in y2's type
+        T2* y2c = y2 + (size_t)r * H;
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const int i = threadIdx.x + j * blockDim.x;
+            if (i < nv) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y2c[4 * i + e] = from_f32<T2>(v[j][e]);
+            }
+        }
+        return;
+    }
     // v holds the new residual row: its norm with w2
     const float mean2 = center2 ? block_sum(sm2, scratch) / (float)H : 0.f;
     float ss2 = 0.f;
@@ -209,12 +221,18 @@ __global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* _
     }
 }
 
-// `w2`, `y2` (optional, with `add` only): also y2 = norm2(y) of the rows just added to, in `y2`'s dtype.
+// `w2`, `y2` (optional, with `add` only): also y2 = norm2(y) of the rows just added to, in `y2`'s dtype; `y2` without `w2`:
+// y2 = y, the rows just added to in `y2`'s dtype (what a half that reads the rows without a norm takes).
+template <typename T2>
+__global__ void rows_as_kernel(const float* __restrict__ x, T2* __restrict__ y, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = from_f32<T2>(x[i]);
+}
 extern "C" int br_layernorm(const float* x, const float* w, void* y, int y_is_bf16, const int* rows, int R, int H,
                             float eps, int center, int add, const float* w2, void* y2, int y2_is_bf16, float eps2,
                             int center2, hipStream_t s) {
     if (R <= 0) return BR_OK;
-    if (H <= 0 || (add && (y_is_bf16 || rows)) || (w2 && (!add || !y2))) return BR_BAD_ARG;
+    if (H <= 0 || (add && (y_is_bf16 || rows)) || (w2 && !y2) || (y2 && !add)) return BR_BAD_ARG;
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
     const bool vec = (H % 4 == 0) && (H / 4 <= 4 * threads) &&
                      (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)w2 | (uintptr_t)y2) % 16 == 0);
@@ -229,6 +247,11 @@ extern "C" int br_layernorm(const float* x, const float* w, void* y, int y_is_bf
     if (add) layernorm_kernel<float, true><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
     else if (y_is_bf16) layernorm_kernel<bf16, false><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps, center);
     else layernorm_kernel<float, false><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
+    if (y2 && !w2) {
+        const size_t n = (size_t)R * H;
+        if (y2_is_bf16) rows_as_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, s>>>((const float*)y, (bf16*)y2, n);
+        else rows_as_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, s>>>((const float*)y, (float*)y2, n);
+    }
     if (w2) {       // widths the one-pass kernel does not take: the second norm as a launch of its own
         if (y2_is_bf16) layernorm_kernel<bf16, false><<<R, threads, 0, s>>>((const float*)y, w2, (bf16*)y2, nullptr, H, eps2, center2);
         else layernorm_kernel<float, false><<<R, threads, 0, s>>>((const float*)y, w2, (float*)y2, nullptr, H, eps2, center2);

@@ -18,9 +18,26 @@
 // The sums of `attend` run over the pages of the seen blocks and then over the pages of the window's
 // tokens, so the order depends on (p, size, pool) only: whole prompts, portions and single tokens give
 // the same bits.
+//
+// Further rules of what a query sees, each a parameter of the three attention kernels: `chunk` > 0 cuts the
+// sequence into runs of `chunk` positions counted from 0 and a query sees no key of an earlier run (beside the
+// window's rule; a window beyond any position leaves the runs alone); `keep` > 0 lets every query also see the
+// sequence's first `keep` tokens, wherever its window begins.  The kept rows that lie before the window are
+// walked first, like the pooled rows.  `softcap` > 0 bounds the scaled scores: s <- softcap tanh(s / softcap).
 #include "common.h"
 
 #define MAX_EPL 8   // head widths up to 64 * MAX_EPL
+
+// The first position a query at p sees by its window and its run of `chunk` positions; both grow with p.
+__device__ __forceinline__ int pwa_lo(int p, int size, int chunk) {
+    int lo = p - size + 1;
+    if (lo < 0) lo = 0;
+    if (chunk > 0) {
+        const int c = (p / chunk) * chunk;
+        if (c > lo) lo = c;
+    }
+    return lo;
+}
 
 // ------------------------------------------------------------------- prepare -------
 // qkv [T, width] float (the product's float sums: queries, keys, and the values from column `v_col0` on, which is
@@ -29,6 +46,12 @@
 // 1 + q_coef ln(floor((p + 1) / q_every) + 1) at position p, behind its norm.
 // vf_role: 0 none, 1 this layer's values are written to `v_first`, 2 values become
 // (1 - lambda) v + lambda v_first.  Tokens of padding sequences (slot < 0) store nothing.
+// `maps` > 1: every query and key head is `maps` vectors of dk side by side (several score maps over the same
+// values), each normed and rotated by itself.  A key row of the cache is then maps * dk wide, and map m of a query
+// head goes out as a row of that width with zeros outside its own dk elements, so that the attention kernels see
+// nq * maps query heads over nkv kv heads whose scores are the maps' own.  `row_ss` [T, 2]: the sums of squares of
+// the token's whole query and key projections (bias included); the norm then runs over the whole projection
+// instead of a head, and `nw_stride` = dk gives every head norm weights of its own (0: one [dk] for all).
 template <typename T>
 __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     const float* __restrict__ qkv, const float* __restrict__ bias, const float* __restrict__ qn_w,
@@ -37,24 +60,33 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     const int* __restrict__ slots, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ q_out, T* __restrict__ storage, float* __restrict__ v_first,
     const float* __restrict__ lambda, int vf_role, int nq, int nkv, int dk, int dv, int page,
-    int write_cache, int width, int v_col0, float q_coef, int q_every) {
+    int write_cache, int width, int v_col0, float q_coef, int q_every, int maps, const float* __restrict__ row_ss,
+    int nw_stride) {
     extern __shared__ float row[];          // [max(dk, dv)]
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const bool is_q = h < nq, is_k = !is_q && h < nq + nkv;
-    const int kvh = is_q ? 0 : (is_k ? h - nq : h - nq - nkv);
+    const int nqs = nq * maps, nks = nkv * maps, kw = maps * dk;     // vectors of dk, and a key row's width
+    const bool is_q = h < nqs, is_k = !is_q && h < nqs + nks;
+    const int sub = is_q ? h : h - nqs;                              // which vector of the queries (keys)
+    const int kvh = is_q ? 0 : (is_k ? sub / maps : h - nqs - nks);
+    const int map = (is_q || is_k) ? sub % maps : 0;
     const int n = (is_q || is_k) ? dk : dv;
-    const int col0 = is_q ? h * dk : (is_k ? nq * dk + kvh * dk : v_col0 + kvh * dv);
+    const int col0 = is_q ? h * dk : (is_k ? nqs * dk + sub * dk : v_col0 + kvh * dv);
     const float* src = qkv + (size_t)t * width + col0;
     const int slot = slots[seq_of_token[t]];
     const int p = pos[t];
     T* dst = nullptr;
-    if (is_q) dst = q_out + ((size_t)t * nq + h) * dk;
-    else if (write_cache && slot >= 0) {
-        const size_t page_elems = (size_t)nkv * page * (dk + dv);
+    if (is_q) {
+        T* qrow = q_out + ((size_t)t * nqs + h) * kw;
+        dst = qrow + map * dk;
+        for (int mm = 0; mm < maps; ++mm)                             // zeros where the other maps' keys lie
+            if (mm != map)
+                for (int i = lane; i < dk; i += 64) qrow[mm * dk + i] = from_f32<T>(0.f);
+    } else if (write_cache && slot >= 0) {
+        const size_t page_elems = (size_t)nkv * page * (kw + dv);
         const int pg = block_table[(size_t)slot * table_stride + p / page];
         T* pb = storage + (size_t)pg * page_elems;
-        dst = is_k ? pb + ((size_t)kvh * page + (p % page)) * dk
-                   : pb + (size_t)nkv * page * dk + (size_t)kvh * dv * page + (p % page);
+        dst = is_k ? pb + ((size_t)kvh * page + (p % page)) * kw + map * dk
+                   : pb + (size_t)nkv * page * kw + (size_t)kvh * dv * page + (p % page);
     }
     const int dst_step = (is_q || is_k) ? 1 : page;      // values lie transposed: channel i of a token at i * page
     float v[MAX_EPL];
@@ -72,7 +104,9 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     if (qk) {
         const float* nw = is_q ? qn_w : kn_w;
         if (nw) {
-            const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
+            const float inv = row_ss ? 1.0f / sqrtf(row_ss[2 * (size_t)t + (is_k ? 1 : 0)] / (float)((is_q ? nqs : nks) * dk) + eps)
+                                     : 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
+            nw += (size_t)sub * nw_stride;
 #pragma unroll
             for (int j = 0; j < MAX_EPL; ++j) {
                 const int i = lane + 64 * j;
@@ -138,6 +172,7 @@ __global__ __launch_bounds__(256) void pwa_values_kernel(
     const int* __restrict__ seq_of_token, const int* __restrict__ slots, const int* __restrict__ block_table,
     int table_stride, T* __restrict__ storage, float* __restrict__ v_first, const float* __restrict__ lambda,
     int vf_role, int n_tokens, int nq, int nkv, int dk, int dv, int page, int width, int v_col0) {
+    // `dk` is the width of a key row of the cache (all maps of a head)
     __shared__ float tile[64][65];
     const int t0 = blockIdx.x * 64, kvh = blockIdx.y, c0 = blockIdx.z * 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -172,40 +207,105 @@ __global__ __launch_bounds__(256) void pwa_values_kernel(
     }
 }
 
+// The sums of squares of a token's whole query projection and of its whole key projection (bias included), for a
+// norm that runs over the projection instead of a head: out [T, 2].  grid (T), 256 threads, a fixed tree per row.
+__global__ __launch_bounds__(256) void pwa_row_ss_kernel(const float* __restrict__ qkv, const float* __restrict__ bias,
+                                                         float* __restrict__ out, int width, int nq_cols, int nk_cols) {
+    __shared__ float scratch[16];
+    const size_t t = blockIdx.x;
+    const float* src = qkv + t * width;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < nq_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sq = fmaf(v, v, sq); }
+    for (int i = nq_cols + threadIdx.x; i < nq_cols + nk_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sk = fmaf(v, v, sk); }
+    sq = block_sum(sq, scratch);
+    sk = block_sum(sk, scratch);
+    if (threadIdx.x == 0) { out[2 * t] = sq; out[2 * t + 1] = sk; }
+}
+
+// `maps`, `row_ss` (scratch float [T, 2] when the norm runs over the whole projection, else null) and `nw_stride`:
+// see the kernel.
 extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* qn_w, const float* kn_w, float eps,
                               const float* cs, const float* sn, int rd, const int* pos, const int* seq_of_token,
                               const int* slots, const int* block_table, int table_stride, void* q_out,
                               void* storage, int is_bf16, float* v_first, const float* lambda, int vf_role,
                               int T, int nq, int nkv, int dk, int dv, int page, int write_cache, int width, int v_from_k,
-                              float q_coef, int q_every, hipStream_t s) {
+                              float q_coef, int q_every, int maps, float* row_ss, int nw_stride, hipStream_t s) {
     if (T <= 0) return BR_OK;
-    const int v_col0 = v_from_k ? nq * dk : nq * dk + nkv * dk;
+    if (maps <= 0 || (maps > 1 && v_from_k) || (nw_stride != 0 && nw_stride != dk)) return BR_BAD_ARG;
+    const int nqs = nq * maps, nks = nkv * maps, kw = maps * dk;
+    const int v_col0 = v_from_k ? nqs * dk : (nqs + nks) * dk;
     if (width < v_col0 + nkv * dv || (v_from_k && dv != dk) || (bias && v_from_k) || q_every < 0) return BR_BAD_ARG;
-    if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL ||
-        rd < 0 || rd > dk || (rd & 1) || page <= 0 || nq + 2 * nkv > 65535 || (rd > 0 && (!cs || !sn)) ||
-        (vf_role && !v_first) || (vf_role == 2 && !lambda) || vf_role < 0 || vf_role > 2)
+    if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || kw > 64 * MAX_EPL || dv > 64 * MAX_EPL ||
+        rd < 0 || rd > dk || (rd & 1) || page <= 0 || nqs + nks + nkv > 65535 || (rd > 0 && (!cs || !sn)) ||
+        (vf_role && !v_first) || (vf_role == 2 && !lambda) || vf_role < 0 || vf_role > 2 || (row_ss && (!qn_w || !kn_w)))
         return BR_BAD_ARG;
+    if (row_ss) {
+        pwa_row_ss_kernel<<<T, 256, 0, s>>>(qkv, bias, row_ss, width, nqs * dk, nks * dk);
+        const int rc0 = br_check_launch();
+        if (rc0 != BR_OK) return rc0;
+    }
     // steps of many tokens that store their values: the values by the tile kernel
     const bool tiled = T >= 256 && write_cache;
-    dim3 grid(T, nq + nkv + (tiled ? 0 : nkv));
+    dim3 grid(T, nqs + nks + (tiled ? 0 : nkv));
     const size_t lds = (size_t)(dk > dv ? dk : dv) * sizeof(float);
     if (is_bf16)
         pwa_prepare_kernel<bf16><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                        block_table, table_stride, (bf16*)q_out, (bf16*)storage, v_first,
-                                                       lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every);
+                                                       lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every,
+                                                       maps, row_ss, nw_stride);
     else
         pwa_prepare_kernel<float><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                         block_table, table_stride, (float*)q_out, (float*)storage,
-                                                        v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every);
+                                                        v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every,
+                                                        maps, row_ss, nw_stride);
     int rc = br_check_launch();
     if (rc != BR_OK || !tiled) return rc;
     dim3 vgrid((T + 63) / 64, nkv, (dv + 63) / 64);
     if (is_bf16)
         pwa_values_kernel<bf16><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (bf16*)storage,
-                                                      v_first, lambda, vf_role, T, nq, nkv, dk, dv, page, width, v_col0);
+                                                      v_first, lambda, vf_role, T, nq, nkv, kw, dv, page, width, v_col0);
     else
         pwa_values_kernel<float><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (float*)storage,
-                                                       v_first, lambda, vf_role, T, nq, nkv, dk, dv, page, width, v_col0);
+                                                       v_first, lambda, vf_role, T, nq, nkv, kw, dv, page, width, v_col0);
+    return br_check_launch();
+}
+
+// ------------------------------------------------ two score maps into one head -----
+// o[t, h, :] = (a1 - lambda a2) / sqrt(mean((a1 - lambda a2)^2) + eps) * scale, where a1 and a2 are the rows of the
+// two maps of head h in `a` [T, nq, 2, dv] (what the attention kernels leave for 2 nq query heads).  `eps` < 0: no
+// norm, o = (a1 - lambda a2) * scale.  A wave a (token, head) row, float arithmetic.  grid (ceil(T nq / 4)), 256.
+template <typename T>
+__global__ __launch_bounds__(256) void pwa_pair_combine_kernel(const T* __restrict__ a, T* __restrict__ o, size_t n_rows, int dv,
+                                                               float lambda, float eps, float scale) {
+    const size_t r = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (r >= n_rows) return;
+    const T* a1 = a + r * 2 * dv;
+    const T* a2 = a1 + dv;
+    float v[MAX_EPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAX_EPL; ++j) {
+        const int i = lane + 64 * j;
+        v[j] = 0.f;
+        if (i < dv) { v[j] = to_f32<T>(a1[i]) - lambda * to_f32<T>(a2[i]); ss = fmaf(v[j], v[j], ss); }
+    }
+    const float mul = eps < 0.f ? scale : scale / sqrtf(wave_sum(ss) / (float)dv + eps);
+#pragma unroll
+    for (int j = 0; j < MAX_EPL; ++j) {
+        const int i = lane + 64 * j;
+        if (i < dv) o[r * dv + i] = from_f32<T>(v[j] * mul);
+    }
+}
+
+extern "C" int br_pwa_pair_combine(const void* a, void* o, int is_bf16, int T, int nq, int dv, float lambda, float eps,
+                                   float scale, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (nq <= 0 || dv <= 0 || dv > 64 * MAX_EPL) return BR_BAD_ARG;
+    const size_t n_rows = (size_t)T * nq;
+    const unsigned blocks = (unsigned)((n_rows + 3) / 4);
+    if (is_bf16) pwa_pair_combine_kernel<bf16><<<blocks, 256, 0, s>>>((const bf16*)a, (bf16*)o, n_rows, dv, lambda, eps, scale);
+    else pwa_pair_combine_kernel<float><<<blocks, 256, 0, s>>>((const float*)a, (float*)o, n_rows, dv, lambda, eps, scale);
     return br_check_launch();
 }
 
@@ -324,7 +424,8 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
     const int* __restrict__ seq_of_token, const int* __restrict__ slots,
     const int* __restrict__ block_table, int table_stride, const T* __restrict__ storage,
     const int* __restrict__ pooled_table, int pooled_stride, const T* __restrict__ pooled,
-    int nq, int nkv, int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
+    int nq, int nkv, int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks,
+    int chunk, int keep, float softcap) {
     extern __shared__ float lds[];
     float* qs = lds;                         // [dk]
     float* ps = qs + dk;                     // [4][64]
@@ -344,11 +445,13 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
     for (int d = threadIdx.x; d < dk; d += 256) qs[d] = to_f32<T>(qr[d]);
     __syncthreads();
     const int p = pos[t];
-    const int lo = (p - size + 1 > 0) ? p - size + 1 : 0;
+    const int lo = pwa_lo(p, size, chunk);
     int seen = 0;
     if (pool > 0 && p - size - pool + 1 >= 0) seen = (p - size - pool + 1) / pool + 1;
     const int far_pages = (seen + page - 1) / page;
-    const int first_page = lo / page, n_pages = far_pages + p / page - first_page + 1;
+    const int kept = keep < lo ? keep : lo;                            // the first tokens that lie before the window
+    const int kept_pages = (kept + page - 1) / page;
+    const int first_page = lo / page, n_pages = far_pages + kept_pages + p / page - first_page + 1;
     const int* bt = block_table + (size_t)slot * table_stride;
     const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
     const size_t page_elems = (size_t)nkv * page * (dk + dv);
@@ -361,11 +464,11 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
     for (int i = 0; i < MAX_EPL; ++i) acc[i] = 0.f;
 
     for (int n = wave; n < n_pages; n += 4) {
-        const bool far = n < far_pages;
-        const int pi = far ? n : first_page + (n - far_pages);         // page index within its unit
+        const bool far = n < far_pages, early = !far && n < far_pages + kept_pages;
+        const int pi = far ? n : (early ? n - far_pages : first_page + (n - far_pages - kept_pages));   // page index within its unit
         const T* base = far ? pooled + (size_t)pt[pi] * page_elems : storage + (size_t)bt[pi] * page_elems;
         const int row0 = pi * page;                                    // first row of the page
-        const int first_ok = far ? 0 : lo, last_ok = far ? seen - 1 : p;
+        const int first_ok = (far || early) ? 0 : lo, last_ok = far ? seen - 1 : (early ? kept - 1 : p);
         float s = -INFINITY;
         for (int j = lane; j < page; j += 64) {                       // pages of 64 rows: one row a lane
             const int key = row0 + j;
@@ -382,6 +485,7 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
                     for (int d = 0; d < dk; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
                 }
                 s = dot * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);
             }
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -439,17 +543,19 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
 extern "C" int br_pwa_attend(const void* q, void* out, int is_bf16, const int* pos, const int* seq_of_token,
                              const int* slots, const int* block_table, int table_stride, const void* storage,
                              const int* pooled_table, int pooled_stride, const void* pooled, int T, int nq, int nkv,
-                             int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks, hipStream_t s) {
+                             int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks,
+                             int chunk, int keep, float softcap, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL || page != 64 ||
-        size <= 0 || pool < 0 || nq > 65535 || (pool > 0 && (!pooled_table || !pooled)))
+        size <= 0 || pool < 0 || nq > 65535 || (pool > 0 && (!pooled_table || !pooled)) || chunk < 0 || keep < 0 || !(softcap >= 0.f))
         return BR_BAD_ARG;
     dim3 grid(T, nq);
     const size_t lds = (size_t)(dk + 256 + 8 + 4 * dv) * sizeof(float);
     // 16-byte loads where every row starts at a multiple of 16 bytes
     const bool vec = is_bf16 ? dk % 8 == 0 : dk % 4 == 0;
 #define PWA_ATT(TT, V) pwa_attend_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)q, (TT*)out, pos, seq_of_token, slots, block_table, \
-        table_stride, (const TT*)storage, pooled_table, pooled_stride, (const TT*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink, sinks)
+        table_stride, (const TT*)storage, pooled_table, pooled_stride, (const TT*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink, sinks, \
+        chunk, keep, softcap)
     if (is_bf16) { if (vec) PWA_ATT(bf16, true); else PWA_ATT(bf16, false); }
     else { if (vec) PWA_ATT(float, true); else PWA_ATT(float, false); }
 #undef PWA_ATT
@@ -495,7 +601,7 @@ __device__ __forceinline__ int pwa_key_of_row(int c) { return 16 * (c >> 4) + 8 
 template <int NBK, int NBV>
 __device__ __forceinline__ void pwa_block(const bf16* __restrict__ kblock, int ks, const bf16* __restrict__ vblock, int vs,
                                           int kb, int limit, int first_ok, int last_ok, int dk, int dv, int c, int g,
-                                          const bf16x8* qf, f32x16* acc_o, float& m, float& lsum, float scale2) {
+                                          const bf16x8* qf, f32x16* acc_o, float& m, float& lsum, float scale2, float cap_in, float cap_out) {
     const bf16* krow = kblock + (size_t)pwa_key_of_row(c) * ks;
     f32x16 s_acc;
 #pragma unroll
@@ -505,6 +611,13 @@ __device__ __forceinline__ void pwa_block(const bf16* __restrict__ kblock, int k
         const int d = s * 16 + 8 * g;
         const bf16x8 kf = (d < dk) ? *(const bf16x8*)(krow + d) : pwa_zero8();
         s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+    }
+    if (cap_out != 0.f) {
+        // bounded scores: cap tanh(s scale / cap), tanh z = 1 - 2 / (exp(2 z) + 1); cap_in = 2 log2(e) scale / cap and
+        // cap_out = cap / scale, so that the multiplication by scale2 below leaves the bounded score in base 2
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            s_acc[r] = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s_acc[r] * cap_in) + 1.0f));
     }
     float sv[16];
     float mx = -INFINITY;
@@ -570,7 +683,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair,
+    int chunk, int keep, float softcap) {
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
@@ -610,6 +724,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     // the two lane halves of a query add their sums at the end: the sink's one goes to the first
     float m = sink ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
+    const bool capped = softcap > 0.f && scale != 0.f;
+    const float cap_in = capped ? 2.0f * PWA_LOG2E * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
     const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
     const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
 
@@ -624,18 +740,28 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
             const int kl = kb % PWA_PAGE;
             const bf16* pg = pooled + (size_t)pt[kb / PWA_PAGE] * page_elems;
             pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, written - kb, 0, seen - 1, dk, dv, c, g,
-                                qf, acc_o, m, lsum, scale2);
+                                qf, acc_o, m, lsum, scale2, cap_in, cap_out);
         }
     }
     const int* bt = block_table + (size_t)slot * table_stride;
-    int lo = pq_min - size + 1;
-    if (lo < 0) lo = 0;
-    const int first_ok = row_ok ? pq - size + 1 : 1, last_ok = row_ok ? pq : 0;
+    const int lo = pwa_lo(pq_min, size, chunk);
+    const int first_ok = row_ok ? pwa_lo(pq, size, chunk) : 1, last_ok = row_ok ? pq : 0;
+    if (keep > 0) {
+        // the sequence's first tokens where they lie before a query's window
+        const int lo_max = pwa_lo(pq_max, size, chunk);
+        const int kept_max = keep < lo_max ? keep : lo_max, kept = row_ok ? (keep < first_ok ? keep : first_ok) : 0;
+        for (int kb = 0; kb < kept_max; kb += 32) {
+            const int kl = kb % PWA_PAGE;
+            const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
+            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, 0, kept - 1, dk, dv, c, g,
+                                qf, acc_o, m, lsum, scale2, cap_in, cap_out);
+        }
+    }
     for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
         const int kl = kb % PWA_PAGE;
         const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
         pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, first_ok, last_ok, dk, dv, c, g,
-                            qf, acc_o, m, lsum, scale2);
+                            qf, acc_o, m, lsum, scale2, cap_in, cap_out);
     }
     lsum += __shfl_xor(lsum, 32, 64);
     if (!row_ok) return;
@@ -668,7 +794,8 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
     const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int cache_heads) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int cache_heads,
+    int chunk, int keep, float softcap) {
     extern __shared__ float lds[];
     const int b = blockIdx.y, kvh = blockIdx.x;
     const int slot = slots[b];
@@ -696,6 +823,8 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     float m = (sink && wave == 0) ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && wave == 0 && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
+    const bool capped = softcap > 0.f && scale != 0.f;
+    const float cap_in = capped ? 2.0f * PWA_LOG2E * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
     // `nkv` blocks of query heads over `cache_heads` kv heads of the cache (more blocks than kv heads: several
     // workgroups read the same rows, each for its own query heads)
     const int ckv = (int)((long long)kvh * cache_heads / nkv);
@@ -704,21 +833,22 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
     int seen = 0;
     if (pool > 0 && pq - size - pool + 1 >= 0) seen = (pq - size - pool + 1) / pool + 1;
     const int far_blocks = (seen + 31) / 32;
-    int lo = pq - size + 1;
-    if (lo < 0) lo = 0;
+    const int lo = pwa_lo(pq, size, chunk);
+    const int kept = keep < lo ? keep : lo;                  // the first tokens that lie before the window
+    const int kept_blocks = (kept + 31) / 32;
     const int kb0 = (lo / 32) * 32;
-    const int n_blocks = far_blocks + (pq - kb0) / 32 + 1;
+    const int n_blocks = far_blocks + kept_blocks + (pq - kb0) / 32 + 1;
     const int* bt = block_table + (size_t)slot * table_stride;
     const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
     for (int n = wave; n < n_blocks; n += PWA_DW) {
-        const bool far = n < far_blocks;
-        const int kb = far ? n * 32 : kb0 + (n - far_blocks) * 32;
+        const bool far = n < far_blocks, early = !far && n < far_blocks + kept_blocks;
+        const int kb = far ? n * 32 : (early ? (n - far_blocks) * 32 : kb0 + (n - far_blocks - kept_blocks) * 32);
         const int kl = kb % PWA_PAGE;
         const bf16* pg = far ? pooled + (size_t)pt[kb / PWA_PAGE] * page_elems : storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
         const int limit = (far ? ctx / pool : ctx) - (kb - kl);
-        const int first_ok = row_ok ? (far ? 0 : lo) : 1, last_ok = row_ok ? (far ? seen - 1 : pq) : 0;
+        const int first_ok = row_ok ? ((far || early) ? 0 : lo) : 1, last_ok = row_ok ? (far ? seen - 1 : (early ? kept - 1 : pq)) : 0;
         pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, limit - kl, first_ok, last_ok, dk, dv, c, g,
-                            qf, acc_o, m, lsum, scale2);
+                            qf, acc_o, m, lsum, scale2, cap_in, cap_out);
     }
     lsum += __shfl_xor(lsum, 32, 64);
     // merge: [wave][2 G lanes] of m and l, [wave][NBV * 16][2 G lanes] of O
@@ -770,7 +900,8 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
 template <int NBK>
 static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStream_t s, const bf16* q, bf16* out, const int* slots,
                                const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
-                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds, int cache_heads) {
+                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds, int cache_heads,
+                               int chunk, int keep, float softcap) {
     // merges beyond 64 KB of LDS (many query heads to a kv head with wide values) are asked for once per kernel
 #define PWA_GO(V) do { \
         auto kern = pwa_decode_kernel<NBK, V>; \
@@ -780,7 +911,7 @@ static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStrea
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
             have = lds; \
         } \
-        kern<<<grid, 64 * PWA_DW, lds, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, cache_heads); \
+        kern<<<grid, 64 * PWA_DW, lds, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, cache_heads, chunk, keep, softcap); \
     } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
@@ -805,20 +936,21 @@ extern "C" int br_pwa_decode_takes(int nq, int nkv, int dk, int dv) {
 extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, const int* ctx_lens, const int* block_table,
                                   int table_stride, const void* storage, const int* pooled_table, int pooled_stride,
                                   const void* pooled, int B, int nq, int nkv, int dk, int dv, int size, int pool, float scale,
-                                  int sink, const float* __restrict__ sinks, int cache_heads, hipStream_t s) {
+                                  int sink, const float* __restrict__ sinks, int cache_heads, int chunk, int keep, float softcap, hipStream_t s) {
     // `nkv` counts the blocks of query heads a workgroup serves; the cache holds `cache_heads` kv heads (0: as many),
     // which `nkv` is a multiple of
     if (B <= 0) return BR_OK;
     if (cache_heads <= 0) cache_heads = nkv;
     if (!br_pwa_decode_takes(nq, nkv, dk, dv) || nkv > 65535 || B > 65535 || size <= 0 || pool < 0 || nkv % cache_heads ||
-        (pool > 0 && (!pooled_table || !pooled)))
+        (pool > 0 && (!pooled_table || !pooled)) || chunk < 0 || keep < 0 || !(softcap >= 0.f))
         return BR_BAD_ARG;
     const int G = nq / nkv;
     dim3 grid(nkv, B);
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
     const size_t head_lds = (size_t)2 * PWA_DW * 2 * G * sizeof(float), per_v = (size_t)PWA_DW * 16 * 2 * G * sizeof(float);
 #define PWA_K(KK) pwa_decode_launch_v<KK>(nbv, grid, per_v, s, (const bf16*)q, (bf16*)out, slots, ctx_lens, block_table, table_stride, \
-                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, head_lds, cache_heads)
+                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, head_lds, cache_heads, \
+                                          chunk, keep, softcap)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);
@@ -840,7 +972,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair,
+    int chunk, int keep, float softcap) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pwa_lds[];
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
@@ -884,6 +1017,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     float m = sink ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
+    const bool capped = softcap > 0.f && scale != 0.f;
+    const float cap_in = capped ? 2.0f * PWA_LOG2E * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
     const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
     const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
 
@@ -891,14 +1026,16 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     auto seen_of = [&](int p) { const int far = p - size - pool + 1; return (pool > 0 && far >= 0) ? far / pool + 1 : 0; };
     const int seen = row_ok ? seen_of(pq) : 0, seen_wave = wave_on ? seen_of(pq_max) : 0;
     const int far_pages = (seen_of(wg_max) + PWA_PAGE - 1) / PWA_PAGE;
-    int wg_lo = wg_min - size + 1;
-    if (wg_lo < 0) wg_lo = 0;
-    int lo_wave = pq_min - size + 1;
-    if (lo_wave < 0) lo_wave = 0;
+    const int wg_lo = pwa_lo(wg_min, size, chunk);
+    const int lo_wave = pwa_lo(pq_min, size, chunk);
     const int first_page = wg_lo / PWA_PAGE;
-    const int n_pages = far_pages + wg_max / PWA_PAGE - first_page + 1;
+    // the sequence's first `keep` tokens where they lie before a query's window: pages of their own in the walk
+    auto kept_of = [&](int p) { const int l = pwa_lo(p, size, chunk); return keep < l ? keep : l; };
+    const int kept = row_ok ? kept_of(pq) : 0, kept_wave = wave_on ? kept_of(pq_max) : 0;
+    const int kept_pages = (kept_of(wg_max) + PWA_PAGE - 1) / PWA_PAGE;
+    const int n_pages = far_pages + kept_pages + wg_max / PWA_PAGE - first_page + 1;
     const int written_far = pool > 0 ? ctx / pool : 0;
-    const int first_ok = row_ok ? pq - size + 1 : 1, last_ok = row_ok ? pq : 0;
+    const int first_ok = row_ok ? pwa_lo(pq, size, chunk) : 1, last_ok = row_ok ? pq : 0;
     const int* bt = block_table + (size_t)slot * table_stride;
     const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
 
@@ -909,7 +1046,9 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const int k_pieces = PWA_PAGE * dk / 8, v_pieces = dv * 8;
     bf16x8 rk[NBK], rv[NBV];
     auto page_of = [&](int n) -> const bf16* {
-        return n < far_pages ? pooled + (size_t)pt[n] * page_elems : storage + (size_t)bt[first_page + (n - far_pages)] * page_elems;
+        if (n < far_pages) return pooled + (size_t)pt[n] * page_elems;
+        if (n < far_pages + kept_pages) return storage + (size_t)bt[n - far_pages] * page_elems;
+        return storage + (size_t)bt[first_page + (n - far_pages - kept_pages)] * page_elems;
     };
     auto fetch = [&](int n) {
         const bf16* pg = page_of(n);
@@ -947,15 +1086,16 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
         if (n + 1 < n_pages) fetch(n + 1);
         const bf16* st = stage0 + (size_t)buf * stage_elems;
         const bf16* sv = st + (size_t)PWA_PAGE * ks;
-        const bool far = n < far_pages;
-        const int page_row0 = (far ? n : first_page + (n - far_pages)) * PWA_PAGE;
+        const bool far = n < far_pages, early = !far && n < far_pages + kept_pages;
+        const int page_row0 = (far ? n : (early ? n - far_pages : first_page + (n - far_pages - kept_pages))) * PWA_PAGE;
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
             const int kb = page_row0 + 32 * hb;
-            const bool mine = wave_on && (far ? kb < seen_wave : (kb + 31 >= lo_wave && kb <= pq_max));     // wave-uniform
+            const bool mine = wave_on && (far ? kb < seen_wave : (early ? kb < kept_wave : (kb + 31 >= lo_wave && kb <= pq_max)));     // wave-uniform
             if (mine)
                 pwa_block<NBK, NBV>(st + (size_t)(32 * hb) * ks, ks, sv + 32 * hb, vs, kb, (far ? written_far : ctx) - kb,
-                                    far ? 0 : first_ok, far ? seen - 1 : last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+                                    (far || early) ? 0 : first_ok, far ? seen - 1 : (early ? kept - 1 : last_ok), dk, dv, c, g, qf, acc_o, m, lsum,
+                                    scale2, cap_in, cap_out);
         }
         if (n + 1 < n_pages) put(buf ^ 1);
         __syncthreads();
@@ -980,7 +1120,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
 template <int NBK>
 static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
                                 const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
-                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
+                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks,
+                                int chunk, int keep, float softcap) {
     // steps that fill a workgroup's 128 rows stage the pages in LDS (key widths in steps of 8 and value widths in steps
     // of 8 that the kernel's pieces cover); shorter ones read their operands straight from the cache
     const int cus = br_device_cus();
@@ -995,8 +1136,8 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
                 if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
                 have = lds; \
             } \
-            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair); \
-        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair); \
+            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap); \
+        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap); \
     } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
@@ -1011,16 +1152,18 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
 extern "C" int br_pwa_prefill_bf16(const void* q, void* out, const int* cu_seqlens, const int* slots, const int* ctx_lens,
                                    const int* block_table, int table_stride, const void* storage, const int* pooled_table,
                                    int pooled_stride, const void* pooled, int B, int max_new, int nq, int nkv, int dk, int dv,
-                                   int size, int pool, float scale, int sink, const float* __restrict__ sinks, hipStream_t s) {
+                                   int size, int pool, float scale, int sink, const float* __restrict__ sinks, int chunk, int keep,
+                                   float softcap, hipStream_t s) {
     if (B <= 0 || max_new <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || nkv > 65535 || B > 65535 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 ||
-        dv % 4 || size <= 0 || pool < 0 || (pool > 0 && (!pooled_table || !pooled)))
+        dv % 4 || size <= 0 || pool < 0 || (pool > 0 && (!pooled_table || !pooled)) || chunk < 0 || keep < 0 || !(softcap >= 0.f))
         return BR_BAD_ARG;
     const int G = nq / nkv;
     dim3 grid((unsigned)(((size_t)max_new * G + 127) / 128), nkv, B);
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
 #define PWA_K(KK) pwa_prefill_launch_v<KK>(nbv, grid, s, (const bf16*)q, (bf16*)out, cu_seqlens, slots, ctx_lens, block_table, table_stride, \
-                                           (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks)
+                                           (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, \
+                                           chunk, keep, softcap)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);

@@ -61,6 +61,112 @@ extern "C" int br_route_topk(const float* scores, const float* bias, int* chosen
     return br_check_launch();
 }
 
+// Routing by sigmoid scores with a choice correction and groups of experts.  s = sigmoid(z); the choice is made on
+// c = s + correction, the shares on s.  With `groups` > 1 the experts form that many runs of E / groups neighbours; a
+// run's score is the sum of its two largest c (of its one, where a run is one expert), only experts of the `keep`
+// best runs can be chosen (the others count as minus infinity), ties to the lower number everywhere.  The shares are
+// the chosen experts' s over their sum (+ 1e-20), times `out_scale`.  grid (T), one wave a token; LDS: E floats.
+__global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restrict__ scores, const float* __restrict__ correction,
+                                                           int* __restrict__ chosen, float* __restrict__ share, int E, int top,
+                                                           int groups, int keep, float out_scale) {
+    extern __shared__ float cs[];           // the choice scores
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float sg[RX_MAX_PER_LANE], z[RX_MAX_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        sg[i] = 0.f;
+        z[i] = -INFINITY;
+        if (e < E) {
+            sg[i] = 1.0f / (1.0f + expf(-scores[(size_t)t * E + e]));
+            z[i] = sg[i] + (correction ? correction[e] : 0.f);
+            cs[e] = z[i];
+        }
+    }
+    if (groups > 1) {
+        __syncthreads();
+        const int per = E / groups;
+        // lane g scores run g + 64 j; the best `keep` runs are taken one after the other
+        float gs[RX_MAX_PER_LANE];
+#pragma unroll
+        for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
+            const int g = lane + 64 * j;
+            gs[j] = -INFINITY;
+            if (g < groups) {
+                float b1 = -INFINITY, b2 = -INFINITY;
+                for (int i = 0; i < per; ++i) {
+                    const float v = cs[g * per + i];
+                    if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) b2 = v;
+                }
+                gs[j] = per > 1 ? b1 + b2 : b1;
+            }
+        }
+        __syncthreads();
+        for (int e = lane; e < E; e += 64) cs[e] = -INFINITY;      // now: minus infinity unless the expert's run is kept
+        __syncthreads();
+        for (int r = 0; r < keep; ++r) {
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+#pragma unroll
+            for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
+                const int g = lane + 64 * j;
+                if (g < groups && gs[j] != -INFINITY && (gs[j] > best || (gs[j] == best && g < at)) ) { best = gs[j]; at = g; }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, WAVE);
+                const int oa = __shfl_xor(at, o, WAVE);
+                if (oa < 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+            }
+            if (at == 0x7fffffff) break;          // fewer runs with a score than `keep`
+#pragma unroll
+            for (int j = 0; j < RX_MAX_PER_LANE; ++j)
+                if (lane + 64 * j == at) gs[j] = -INFINITY;
+            for (int i = lane; i < per; i += 64) cs[at * per + i] = 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && cs[e] != 0.f) z[i] = -INFINITY;
+        }
+    }
+    float total = 0.f, mine = 0.f;
+    for (int s = 0; s < top; ++s) {
+        float best = -INFINITY, bs = 0.f;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && (z[i] > best || (z[i] == best && e < at))) { best = z[i]; at = e; bs = sg[i]; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, WAVE), os = __shfl_xor(bs, o, WAVE);
+            const int oa = __shfl_xor(at, o, WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; bs = os; }
+        }
+        if (at >= E) { at = s; bs = 0.f; }        // scores that compare with nothing (a padding row's): any expert will do
+        total += bs;
+        if (lane == s) mine = bs;                 // lane s keeps slot s's score
+        if (lane == 0) chosen[(size_t)t * top + s] = at;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i)
+            if (lane + 64 * i == at) z[i] = -INFINITY;
+    }
+    if (lane < top) share[(size_t)t * top + lane] = mine / (total + 1e-20f) * out_scale;
+}
+
+extern "C" int br_route_sigmoid(const float* scores, const float* correction, int* chosen, float* share, int T, int E, int top,
+                                int groups, int keep, float out_scale, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (E <= 0 || E > 64 * RX_MAX_PER_LANE || top <= 0 || top > E || top > 64 || groups <= 0 || E % groups ||
+        (groups > 1 && (keep <= 0 || keep > groups)))
+        return BR_BAD_ARG;
+    route_sigmoid_kernel<<<T, 64, (size_t)E * sizeof(float), s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    return br_check_launch();
+}
+
 template <typename T> struct rx_vec;
 template <> struct rx_vec<float> { static constexpr int N = 4; typedef f32x4 type; };
 template <> struct rx_vec<bf16> { static constexpr int N = 8; typedef bf16x8 type; };

@@ -113,7 +113,8 @@ def layernorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float, r
               center: bool = True, add: bool = False, then=None) -> None:
     """out = norm(x) * w, or out += norm(x) * w with `add` (float `out`); `center` False: the RMS norm.
     `then` = (w2, out2, eps2, center2), with `add` only: the rows just added to are normed once more,
-    out2 = norm2(out) * w2, in the same kernel."""
+    out2 = norm2(out) * w2, in the same kernel; with w2 None out2 takes the rows just added to as they are, in its
+    own dtype (for a reader that takes the rows without a norm)."""
     _dev("layernorm", x, w, out, rows)
     H = x.shape[-1]
     R = out.shape[0]
@@ -130,7 +131,7 @@ def layernorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float, r
     if then is not None:
         w2, out2, eps2, center2 = then
         _dev("layernorm", w2, out2)
-        _req(add and w2.dtype == torch.float32 and w2.numel() == H and out2.shape == (R, H)
+        _req(add and (w2 is None or (w2.dtype == torch.float32 and w2.numel() == H)) and out2.shape == (R, H)
              and out2.data_ptr() not in (x.data_ptr(), out.data_ptr()), "layernorm: the second norm takes float weights [H] "
              "and rows [R, H] of their own, behind an add")
     f = _fn("elementwise", "br_layernorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, c_int, c_int, _P, _P, c_int,
@@ -540,27 +541,39 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
                 rotary_dim: int, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
                 block_table: torch.Tensor, q_out: torch.Tensor, unit: torch.Tensor, v_first: Optional[torch.Tensor],
                 mix: Optional[torch.Tensor], v_role: int, nq: int, nkv: int, dk: int, dv: int, page: int,
-                write_cache: bool, values_from_keys: bool = False, q_temp_coef: float = 0.0, q_temp_every: int = 0) -> None:
+                write_cache: bool, values_from_keys: bool = False, q_temp_coef: float = 0.0, q_temp_every: int = 0,
+                maps: int = 1, row_ss: Optional[torch.Tensor] = None) -> None:
     """Float projection sums [T, nq*dk + nkv*dk + nkv*dv (+ more columns that are not read)] -> queries (normed,
     rotated) in `q_out` and the tokens' keys (normed, rotated) and values in their cache pages.  `v_role` 1 leaves
     the values in `v_first`, 2 mixes them with it by the scalar `mix`.  `values_from_keys`: there are no value
     columns, the keys' sums as projected (before norm and rotation) are the values.  `q_temp_every` > 0: the query
-    at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) behind its norm."""
+    at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) behind its norm.
+    `maps` > 1: every query and key head is `maps` vectors of dk side by side, each normed and rotated by itself; the
+    cache's key rows are maps * dk wide and `q_out` is [T, nq * maps rows of maps * dk], every row one map's query with
+    zeros where the other maps' keys lie (the attention kernels then take nq * maps query heads of maps * dk).  `row_ss`
+    (float scratch [T, 2]): the norm runs over the token's whole query (key) projection instead of over a head, with
+    weights for the whole projection (`q_norm` [nq * maps * dk], `k_norm` [nkv * maps * dk])."""
     _dev("pwa_prepare", qkv, bias, q_norm, k_norm, cos, sin, positions, seq_of_token, slots, block_table, q_out, unit,
-         v_first, mix)
+         v_first, mix, row_ss)
     T = qkv.shape[0]
-    width = nq * dk + nkv * dk + (0 if values_from_keys else nkv * dv)
+    _req(maps >= 1 and (maps == 1 or not values_from_keys), "pwa_prepare: one or more maps; keys that serve as values have one")
+    nqs, nks, kw = nq * maps, nkv * maps, maps * dk
+    width = nqs * dk + nks * dk + (0 if values_from_keys else nkv * dv)
     _req(qkv.dtype == torch.float32 and qkv.dim() == 2 and qkv.shape[1] >= width,
          "pwa_prepare: projections must be float32 [T, nq*dk + nkv*(dk+dv) or more]")
     _req(not values_from_keys or (dv == dk and bias is None), "pwa_prepare: values taken from the keys have their width and no bias")
     _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "pwa_prepare: bias float32 of the projections' width")
     _req(q_temp_every >= 0, "pwa_prepare: the query temperature's period must not be negative")
-    for nw in (q_norm, k_norm):
-        _req(nw is None or (nw.dtype == torch.float32 and nw.numel() == dk), "pwa_prepare: norm weights float32 [dk]")
+    whole = row_ss is not None
+    for nw, heads in ((q_norm, nqs), (k_norm, nks)):
+        _req(nw is None or (nw.dtype == torch.float32 and nw.numel() == (heads * dk if whole else dk)),
+             "pwa_prepare: norm weights float32 [dk], or of the whole projection with a norm over it")
+    _req(not whole or (row_ss.dtype == torch.float32 and row_ss.numel() >= 2 * T and q_norm is not None and k_norm is not None),
+         "pwa_prepare: a norm over the whole projection takes float scratch [T, 2] and weights for queries and keys")
     _req(positions.numel() >= T and seq_of_token.numel() >= T, "pwa_prepare: positions shorter than tokens")
     _req(block_table.dim() == 2 and block_table.dtype == torch.int32, "pwa_prepare: block table int32 [slots, pages]")
-    _req(q_out.shape == (T, nq * dk) and q_out.dtype == unit.dtype, "pwa_prepare: q_out [T, nq*dk] of the cache's dtype")
-    _pwa_unit("pwa_prepare", unit, nkv, dk, dv, page)
+    _req(q_out.shape == (T, nqs * kw) and q_out.dtype == unit.dtype, "pwa_prepare: q_out [T, nq*maps*maps*dk] of the cache's dtype")
+    _pwa_unit("pwa_prepare", unit, nkv, kw, dv, page)
     if rotary_dim:
         _req(cos is not None and sin is not None and cos.dtype == sin.dtype == torch.float32
              and cos.numel() >= T * (rotary_dim // 2) and sin.numel() >= T * (rotary_dim // 2), "pwa_prepare: rotary tables float32 [T, rotary_dim/2]")
@@ -569,12 +582,26 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
              "pwa_prepare: v_first float32 [T, nkv*dv]")
         _req(v_role != 2 or (mix is not None and mix.dtype == torch.float32 and mix.numel() == 1), "pwa_prepare: mix is one float")
     f = _fn("pooled_attention", "br_pwa_prepare",
-            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 10 + [c_float, c_int, _P])
+            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 10 + [c_float, c_int, c_int, _P, c_int, _P])
     _check(f(_ptr(qkv), _ptr(bias), _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(cos), _ptr(sin), int(rotary_dim),
              _ptr(positions), _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(q_out),
              _ptr(unit), _is_bf16(unit, "pwa_prepare"), _ptr(v_first), _ptr(mix), int(v_role), T, nq, nkv, dk, dv, page,
              int(write_cache), int(qkv.shape[1]), int(bool(values_from_keys)), float(q_temp_coef), int(q_temp_every),
-             _stream()), "pwa_prepare")
+             int(maps), _ptr(row_ss), dk if whole else 0, _stream()), "pwa_prepare")
+
+
+def pwa_pair_combine(a: torch.Tensor, out: torch.Tensor, nq: int, dv: int, factor: float, eps: Optional[float],
+                     scale: float = 1.0) -> None:
+    """Two score maps a head into one output: a [T, nq*2*dv] holds, head by head, the rows a1 and a2 that attention left
+    for the head's two maps; out[t, h] = (a1 - factor a2) / sqrt(mean((a1 - factor a2)^2) + eps) * scale over the head's
+    dv values (no weight; `eps` None: no norm)."""
+    _dev("pwa_pair_combine", a, out)
+    T = a.shape[0]
+    _req(a.shape == (T, nq * 2 * dv) and out.shape == (T, nq * dv) and a.dtype == out.dtype, "pwa_pair_combine: a [T, nq*2*dv], out [T, nq*dv]")
+    _req(0 < dv <= 512 and (eps is None or eps >= 0), "pwa_pair_combine: value widths up to 512, eps not negative")
+    f = _fn("pooled_attention", "br_pwa_pair_combine", [_P, _P, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P])
+    _check(f(_ptr(a), _ptr(out), _is_bf16(a, "pwa_pair_combine"), T, nq, dv, float(factor), -1.0 if eps is None else float(eps),
+             float(scale), _stream()), "pwa_pair_combine")
 
 
 def pwa_gate(o: torch.Tensor, gate: torch.Tensor, nq: int, dv: int, per_head: bool, scale: float = 1.0) -> None:
@@ -620,8 +647,11 @@ def _sinks(name: str, sinks: Optional[torch.Tensor], nq: int) -> c_void_p:
 def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
                block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
                pooled: Optional[torch.Tensor], nq: int, nkv: int, dk: int, dv: int, page: int, size: int, pool: int,
-               scale: float, sink: bool, sinks: Optional[torch.Tensor] = None) -> None:
-    """One wave per (query, head), float arithmetic: the window's tokens and the pooled blocks before it."""
+               scale: float, sink: bool, sinks: Optional[torch.Tensor] = None, chunk: int = 0, keep: int = 0,
+               softcap: float = 0.0) -> None:
+    """One wave per (query, head), float arithmetic: the window's tokens and the pooled blocks before it.  `chunk` > 0:
+    a query sees no key before its own run of `chunk` positions (counted from 0); `keep` > 0: it also sees the sequence's
+    first `keep` tokens; `softcap` > 0: scores become softcap * tanh(score / softcap)."""
     _dev("pwa_attend", q, out, positions, seq_of_token, slots, block_table, unit, pooled_table, pooled)
     T = q.shape[0]
     _req(q.shape == (T, nq * dk) and out.shape == (T, nq * dv) and q.dtype == out.dtype == unit.dtype,
@@ -631,11 +661,12 @@ def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_attend: pooled unit missing")
         _pwa_unit("pwa_attend", pooled, nkv, dk, dv, page)
     f = _fn("pooled_attention", "br_pwa_attend",
-            [_P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, _P])
+            [_P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, c_int, c_int, c_float, _P])
     _check(f(_ptr(q), _ptr(out), _is_bf16(q, "pwa_attend"), _ptr(positions), _ptr(seq_of_token), _ptr(slots),
              _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
              pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), T, nq, nkv, dk, dv, page, int(size),
-             int(pool), float(scale), int(sink), _sinks("pwa_attend", sinks, nq), _stream()), "pwa_attend")
+             int(pool), float(scale), int(sink), _sinks("pwa_attend", sinks, nq), int(chunk), int(keep), float(softcap),
+             _stream()), "pwa_attend")
 
 
 def pwa_prefill_takes(dtype: torch.dtype, dk: int, dv: int, page: int) -> bool:
@@ -646,7 +677,8 @@ def pwa_prefill_takes(dtype: torch.dtype, dk: int, dv: int, page: int) -> bool:
 def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor,
                      block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
                      pooled: Optional[torch.Tensor], B: int, max_new: int, nq: int, nkv: int, dk: int, dv: int, page: int,
-                     size: int, pool: int, scale: float, sink: bool, sinks: Optional[torch.Tensor] = None) -> None:
+                     size: int, pool: int, scale: float, sink: bool, sinks: Optional[torch.Tensor] = None, chunk: int = 0,
+                     keep: int = 0, softcap: float = 0.0) -> None:
     """Steps of several tokens per sequence on the matrix cores: the same sums as `pwa_attend`, bfloat16 operands,
     float scores and softmax, the weights rounded to bfloat16 for the second product."""
     _dev("pwa_prefill_bf16", q, out, cu_seqlens, slots, ctx_lens, block_table, unit, pooled_table, pooled)
@@ -661,10 +693,11 @@ def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tenso
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_prefill_bf16: pooled unit missing")
         _pwa_unit("pwa_prefill_bf16", pooled, nkv, dk, dv, page)
     f = _fn("pooled_attention", "br_pwa_prefill_bf16",
-            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, _P])
+            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, c_int, c_int, c_float, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit),
              _ptr(pooled_table), pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, max_new, nq, nkv, dk, dv,
-             int(size), int(pool), float(scale), int(sink), _sinks("pwa_prefill_bf16", sinks, nq), _stream()), "pwa_prefill_bf16")
+             int(size), int(pool), float(scale), int(sink), _sinks("pwa_prefill_bf16", sinks, nq), int(chunk), int(keep),
+             float(softcap), _stream()), "pwa_prefill_bf16")
 
 
 def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, page: int) -> bool:
@@ -679,7 +712,8 @@ def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, pa
 def pwa_decode_bf16(q: torch.Tensor, out: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor, block_table: torch.Tensor,
                     unit: torch.Tensor, pooled_table: Optional[torch.Tensor], pooled: Optional[torch.Tensor], B: int, nq: int,
                     nkv: int, dk: int, dv: int, page: int, size: int, pool: int, scale: float, sink: bool,
-                    sinks: Optional[torch.Tensor] = None, cache_heads: int = 0) -> None:
+                    sinks: Optional[torch.Tensor] = None, cache_heads: int = 0, chunk: int = 0, keep: int = 0,
+                    softcap: float = 0.0) -> None:
     """Steps of one token per sequence on the matrix cores (row b of q is sequence b's token): a workgroup per
     (kv head, sequence) serves all query heads of the kv head.  `cache_heads` (0: nkv): the kv heads the cache holds
     when `nkv` is a multiple of them: the query heads of one cache head are then dealt to several workgroups (many
@@ -694,10 +728,11 @@ def pwa_decode_bf16(q: torch.Tensor, out: torch.Tensor, slots: torch.Tensor, ctx
     if pool:
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_decode_bf16: pooled unit missing")
         _pwa_unit("pwa_decode_bf16", pooled, held, dk, dv, page)
-    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P, c_int, _P])
+    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P, c_int, c_int, c_int, c_float, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
              pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, nq, nkv, dk, dv, int(size), int(pool),
-             float(scale), int(sink), _sinks("pwa_decode_bf16", sinks, nq), int(held), _stream()), "pwa_decode_bf16")
+             float(scale), int(sink), _sinks("pwa_decode_bf16", sinks, nq), int(held), int(chunk), int(keep), float(softcap),
+             _stream()), "pwa_decode_bf16")
 
 
 # ------------------------------------------------------ gated linear recurrence -----
@@ -919,6 +954,25 @@ def dr_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gb: Optional[torc
              _ptr(cu_seqlens), _ptr(slots), B, H, G, d, e, int(gb is not None), int(bool(silu)), _stream()), "dr_scan")
 
 
+def dr_rotate_rows(q: torch.Tensor, k: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
+                   heads: int, d: int, q_mul: float = 1.0, k_mul: float = 1.0) -> None:
+    """q and k, float views [T, heads * d] with rows equally far apart, turned in place by their tokens' positions
+    (cos, sin float [T, rotary_dim / 2]; channel i < rotary_dim / 2 of a head pairs with channel i + rotary_dim / 2, the
+    channels from rotary_dim on pass), then multiplied by `q_mul` and `k_mul`."""
+    _dev("dr_rotate_rows", cos, sin)
+    T = q.shape[0]
+    for name, t in (("q", q), ("k", k)):
+        _req(t.is_cuda and t.dtype == torch.float32 and t.shape == (T, heads * d) and t.stride(1) == 1, f"dr_rotate_rows: {name} float32 [T, heads*d]")
+    _req(T <= 1 or q.stride(0) == k.stride(0), "dr_rotate_rows: q and k rows equally far apart")
+    _req(0 <= rotary_dim <= d and rotary_dim % 2 == 0, "dr_rotate_rows: an even number of rotated channels, at most a head's")
+    if rotary_dim:
+        _req(cos is not None and sin is not None and cos.dtype == sin.dtype == torch.float32
+             and cos.numel() >= T * (rotary_dim // 2) and sin.numel() >= T * (rotary_dim // 2), "dr_rotate_rows: rotary tables float32 [T, rotary_dim/2]")
+    f = _fn("delta_rule", "br_dr_rotate_rows", [_P, _P, c_size_t, _P, _P, c_int, c_int, c_int, c_int, c_float, c_float, _P])
+    _check(f(_ptr(q), _ptr(k), q.stride(0) if T > 1 else heads * d, _ptr(cos), _ptr(sin), int(rotary_dim), T, heads, d,
+             float(q_mul), float(k_mul), _stream()), "dr_rotate_rows")
+
+
 def silu_rows(x: torch.Tensor) -> None:
     """x <- silu(x) in place: a float view [T, n] whose rows may be strided (some columns of a projection's sums)."""
     _req(x.is_cuda and x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "silu_rows: a float32 view [T, n] with dense rows")
@@ -1019,6 +1073,26 @@ def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch
     _req(0 < top <= min(E, 64) and E <= 512, f"route_topk: {top} of {E} experts is outside the kernel's sizes (512 experts, 64 chosen)")
     f = _fn("routed_experts", "br_route_topk", [_P, _P, _P, _P, c_int, c_int, c_int, c_float, _P])
     _check(f(_ptr(scores), _ptr(bias), _ptr(chosen), _ptr(share), T, E, top, float(out_scale), _stream()), "route_topk")
+
+
+def route_sigmoid(scores: torch.Tensor, correction: Optional[torch.Tensor], chosen: torch.Tensor, share: torch.Tensor, top: int,
+                  groups: int = 1, keep: int = 1, out_scale: float = 1.0) -> None:
+    """scores float [T, E]: s = sigmoid(scores); the `top` experts with the largest s + correction per row (ties to the
+    lower number) into chosen int32 [T, top], their s over the chosen ones' sum (+ 1e-20) times `out_scale` into share
+    float [T, top].  `groups` > 1: the experts form that many runs of neighbours, a run scores the sum of its two largest
+    s + correction, and only experts of the `keep` best runs can be chosen."""
+    _dev("route_sigmoid", scores, correction, chosen, share)
+    T, E = scores.shape
+    _req(scores.dtype == torch.float32 and (correction is None or (correction.dtype == torch.float32 and correction.numel() == E)),
+         "route_sigmoid: float32 scores and correction")
+    _req(chosen.dtype == torch.int32 and chosen.shape == (T, top) and share.dtype == torch.float32 and share.shape == (T, top),
+         "route_sigmoid: chosen int32 and share float32 [T, top]")
+    _req(0 < top <= min(E, 64) and E <= 512, f"route_sigmoid: {top} of {E} experts is outside the kernel's sizes (512 experts, 64 chosen)")
+    _req(groups >= 1 and E % groups == 0 and (groups == 1 or (1 <= keep <= groups and keep * (E // groups) >= top)),
+         f"route_sigmoid: {groups} runs of experts of which {keep} are kept cannot give {top} of {E} experts")
+    f = _fn("routed_experts", "br_route_sigmoid", [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(scores), _ptr(correction), _ptr(chosen), _ptr(share), T, E, top, int(groups), int(keep), float(out_scale),
+             _stream()), "route_sigmoid")
 
 
 def experts_up(h: torch.Tensor, w_gu: torch.Tensor, chosen: torch.Tensor, y: torch.Tensor) -> None:

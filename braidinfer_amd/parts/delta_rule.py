@@ -13,7 +13,10 @@ multiplied by a weight [e] shared by the heads and by silu(W_g n) [H, e], and pr
 
 Lightning attention (linear attention with a fixed decay per head): q = silu(W_q n), k = silu(W_k n) (H heads of d),
 v = silu(W_v n) (H of e); S <- decay_h S + k v^T, o = S^T q, no other scale.  The concatenated heads are RMS-normed
-together with a weight [H e], multiplied by sigmoid(W_g n) and projected by W_o.
+together with a weight [H e], multiplied by sigmoid(W_g n) and projected by W_o.  Parameters make the same mixer a
+retention layer: `activation` None (q, k, v as projected), `position` (a rotary encoding that turns q and k by the
+token's position before the sum), `key_scale` (k times a constant behind the rotation), `norm` "head" (every head's o
+divided by its own root mean square) with or without weights, `gate` "silu".
 
 What a sequence keeps is fixed in size and float in both precisions, in its slot of the cache's state area
 (`StateNeed`): S per head (zero at first, laid out as the scan kernel's lanes hold it) and, for the convolution, the
@@ -32,7 +35,7 @@ from .. import kernels as K
 from ..cache import StateNeed
 from ..errors import ConfigError, StepError
 from ..weights import TensorSpec
-from .base import Mixer, MixerContext, Runtime, register_part
+from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
 from .gated_recurrence import HGRN2, pieces_for
 from .linear import fused_layout, linear, stream_layout
 
@@ -128,34 +131,58 @@ class LightningAttention(Mixer):
     MIN_PIECE = 128          # tokens: shorter pieces do not pay for the second walk
 
     def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, decay: Sequence[float], norm_eps: float,
-                 out_scale: float = 1.0, names: Optional[Dict[str, str]] = None):
+                 out_scale: float = 1.0, names: Optional[Dict[str, str]] = None, activation: Optional[str] = "silu",
+                 position: Optional[str] = None, key_scale: float = 1.0, norm: str = "all", norm_weight: bool = True,
+                 gate: str = "sigmoid"):
         if num_heads <= 0 or not 0 < key_dim <= 512 or not 0 < value_dim <= 512:
             raise ConfigError(f"lightning attention: {num_heads} heads of {key_dim} key and {value_dim} value channels "
                               "(all positive, widths at most 512)")
+        if activation not in (None, "silu") or norm not in ("all", "head") or gate not in ("sigmoid", "silu"):
+            raise ConfigError(f"lightning attention: activation None or 'silu', norm 'all' or 'head', gate 'sigmoid' or 'silu'; "
+                              f"got {activation!r}, {norm!r}, {gate!r}")
         if len(decay) != num_heads:
             raise ConfigError(f"lightning attention: {len(decay)} decays for {num_heads} heads")
         self.H, self.nh, self.d, self.e = int(hidden_size), int(num_heads), int(key_dim), int(value_dim)
         self.decay_values = [float(g) for g in decay]
         self.eps, self.out_scale = float(norm_eps), float(out_scale)
         self.names = dict(self.NAMES, **(names or {}))
+        self.silu, self.position, self.key_scale = activation == "silu", position, float(key_scale)
+        self.norm_per_head, self.norm_weight, self.gate_sigmoid = norm == "head", bool(norm_weight), gate == "sigmoid"
+        self._expects_tables = False
         self.w_in = self.w_o = self.decay = self.norm_w = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         n, hd, he = self.names, self.nh * self.d, self.nh * self.e
-        return [TensorSpec(prefix + n["q"], (hd, self.H)), TensorSpec(prefix + n["k"], (hd, self.H)),
-                TensorSpec(prefix + n["v"], (he, self.H)), TensorSpec(prefix + n["g"], (he, self.H)),
-                TensorSpec(prefix + n["norm"], (he,), kind="vector", init="ones"),
-                TensorSpec(prefix + n["o"], (self.H, he))]
+        out = [TensorSpec(prefix + n["q"], (hd, self.H)), TensorSpec(prefix + n["k"], (hd, self.H)),
+               TensorSpec(prefix + n["v"], (he, self.H)), TensorSpec(prefix + n["g"], (he, self.H))]
+        if self.norm_weight:
+            out.append(TensorSpec(prefix + n["norm"], (he,), kind="vector", init="ones"))
+        return out + [TensorSpec(prefix + n["o"], (self.H, he))]
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
         n = self.names
         self.w_in = fused_layout([tensors[prefix + n[x]] for x in ("q", "k", "v", "g")], rt)
-        self.w_o = stream_layout(tensors[prefix + n["o"]], rt)
+        w_o = tensors[prefix + n["o"]]
+        if not self.norm_weight and self.out_scale != 1.0:          # no norm weight to carry the multiplier: the matrix does
+            w_o = (w_o.to(torch.float32) * self.out_scale).to(w_o.dtype)
+        self.w_o = stream_layout(w_o, rt)
         decay = rt.empty((self.nh,), torch.float32)
         decay.copy_(torch.tensor(self.decay_values, dtype=torch.float32))
         self.decay = decay
-        self.norm_w = rt.own(tensors[prefix + n["norm"]].to(torch.float32).reshape(-1) * self.out_scale)
+        if self.norm_weight:
+            self.norm_w = rt.own(tensors[prefix + n["norm"]].to(torch.float32).reshape(-1) * self.out_scale)
+
+    def check_positions(self, encodings) -> None:
+        if self.position is None:
+            return
+        enc = encodings.get(self.position)
+        if enc is None or getattr(enc, "gives", None) != "rotary":
+            raise ConfigError(f"lightning attention asks for the rotary encoding {self.position!r}, the model has {sorted(encodings)}")
+        if enc.rotary_dim > self.d or getattr(enc, "pairing", "half") != "half":
+            raise ConfigError(f"lightning attention: the encoding {self.position!r} rotates {enc.rotary_dim} elements in "
+                              f"{getattr(enc, 'pairing', None)!r} pairs; this mixer takes up to {self.d} in 'half' pairs")
+        self._expects_tables = True
 
     def state_need(self) -> StateNeed:
         return StateNeed(tuple(K.glr_state_shape(self.nh, self.d, self.e)), torch.float32)
@@ -168,6 +195,18 @@ class LightningAttention(Mixer):
         rows = step.ws.get("la_rows", (T, 2 * hd + 2 * he), torch.float32)
         linear(h, self.w_in, rows, step.ws)
         o = step.ws.get("la_o", (T, he), torch.float32)
+        silu = self.silu
+        if self._expects_tables or self.key_scale != 1.0:
+            # q and k turned by the position and the key scaled, in place on the float sums (behind the activation)
+            tables = step.position_data.get(self.position) if self.position else None
+            if self._expects_tables and not isinstance(tables, RotaryTables):
+                raise StepError(f"lightning attention: the position encoding {self.position!r} gave {type(tables).__name__}, "
+                                "rotary tables were expected")
+            if silu:
+                K.silu_rows(rows[:, :2 * hd + he])
+                silu = False
+            K.dr_rotate_rows(rows[:, :hd], rows[:, hd:2 * hd], tables.cos if tables else None, tables.sin if tables else None,
+                             tables.rotary_dim if tables else 0, nh, d, 1.0, self.key_scale)
         pieces = pieces_for(step, nh * -(-e // 16), self.MIN_PIECE)
         if pieces > 1:
             # long prompts: the recurrence is linear in the state, so every sequence is cut into pieces that are walked
@@ -175,15 +214,19 @@ class LightningAttention(Mixer):
             cu, numbers = HGRN2._piece_arrays(step, pieces)
             piece_state = step.ws.get("la_piece_state", (step.n_seqs * pieces,) + tuple(K.glr_state_shape(nh, d, e)), torch.float32)
             # two walks by many workgroups a head: the activation once, ahead of them
-            K.silu_rows(rows[:, :2 * hd + he])
+            if silu:
+                K.silu_rows(rows[:, :2 * hd + he])
             K.dr_scan_pieces(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], self.decay, o, ctx.state, step.slots,
                              cu, numbers, piece_state, step.n_seqs, pieces, nh, d, e, silu=False)
         else:
             K.dr_scan(rows[:, :hd], rows[:, hd:2 * hd], rows[:, 2 * hd:2 * hd + he], None, self.decay, o, ctx.state,
-                      step.cu_seqlens, step.slots, step.n_seqs, nh, nh, d, e, silu=True)
+                      step.cu_seqlens, step.slots, step.n_seqs, nh, nh, d, e, silu=silu)
         y = step.ws.get("la_y", (T, he), self.rt.dtype)
-        # all heads normed together: one "head" of H e channels
-        K.head_norm_gate(o, self.norm_w, rows[:, 2 * hd + he:], y, 1, he, self.eps, gate_sigmoid=True)
+        if self.norm_per_head:
+            K.head_norm_gate(o, self.norm_w, rows[:, 2 * hd + he:], y, nh, e, self.eps, gate_sigmoid=self.gate_sigmoid)
+        else:
+            # all heads normed together: one "head" of H e channels
+            K.head_norm_gate(o, self.norm_w, rows[:, 2 * hd + he:], y, 1, he, self.eps, gate_sigmoid=self.gate_sigmoid)
         linear(y, self.w_o, x, step.ws, accumulate=True)
 
 

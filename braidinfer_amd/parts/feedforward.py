@@ -9,7 +9,11 @@ the products' float sums.
 Routed experts: router scores z = W_r n + b_r in float; a token takes the `top` experts with the largest scores
 (ties to the lower number), weighted by the softmax over those scores only (which is also the softmax over all experts divided by the chosen
 ones' sum), and x += sum_s share_s expert_s(n)
-with an expert W_d (silu(W_g n) * (W_u n)) without biases.  The reference has neither."""
+with an expert W_d (silu(W_g n) * (W_u n)) without biases.  `scoring` "sigmoid" routes otherwise: scores s = sigmoid(z);
+the choice is made on s + a learnt correction per expert, among the experts of the best `groups_keep` of `groups`
+equal runs of neighbouring experts (a run scores the sum of its two largest corrected scores); the shares are the
+chosen experts' s over their sum.  `shared_size` adds a gated unit of that inner width that every token passes.  The
+reference has neither."""
 from __future__ import annotations
 
 import os
@@ -117,7 +121,8 @@ class RoutedExperts(FeedForward):
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = True,
-                 names: Optional[Dict[str, str]] = None, out_scale: float = 1.0):
+                 names: Optional[Dict[str, str]] = None, out_scale: float = 1.0, scoring: str = "softmax",
+                 groups: int = 1, groups_keep: int = 1, shared_size: int = 0):
         """`names`: "expert" with {e} for the expert's number (the prefix of its three matrices "gate", "up", "down"),
         "router", "router_bias".  `out_scale` multiplies what is added to the residual rows (it rides on the shares)."""
         self.out_scale = float(out_scale)
@@ -125,9 +130,22 @@ class RoutedExperts(FeedForward):
         if self.I <= 0 or not 0 < self.top <= self.E or self.E > 512 or self.top > 64:
             raise ConfigError(f"routed experts: {top} of {num_experts} experts of inner width {intermediate_size} "
                               "(at most 512 experts, 64 chosen)")
-        self.router_bias = bool(router_bias)
+        if scoring not in ("softmax", "sigmoid"):
+            raise ConfigError(f"routed experts: scoring is 'softmax' or 'sigmoid', got {scoring!r}")
+        self.sigmoid = scoring == "sigmoid"
+        self.groups, self.groups_keep, self.shared_size = int(groups), int(groups_keep), int(shared_size or 0)
+        if self.groups < 1 or self.E % self.groups or (self.groups > 1 and not self.sigmoid) or self.shared_size < 0 or \
+                (self.groups > 1 and not (1 <= self.groups_keep <= self.groups and self.groups_keep * (self.E // self.groups) >= self.top)):
+            raise ConfigError(f"routed experts: {groups} runs of experts of which {groups_keep} are kept must divide the "
+                              f"{num_experts} experts (sigmoid scoring) and leave {top} to choose")
+        self.router_bias = bool(router_bias) and not self.sigmoid
         self.names = dict({"expert": "e{e}.", "gate": "gate", "up": "up", "down": "down", "router": "router",
-                           "router_bias": "router.b"}, **(names or {}))
+                           "router_bias": "router.b", "correction": "correction", "shared": "shared."}, **(names or {}))
+        self.shared = None
+        if self.shared_size:
+            sh = self.names["shared"]
+            self.shared = SwiGLU(self.H, self.shared_size, names={k: sh + self.names[k] for k in ("gate", "up", "down")})
+        self.correction = None
         self.w_gu = self.w_down = self.w_router = self.b_router = None
 
     def _expert(self, prefix: str, e: int, what: str) -> str:
@@ -142,6 +160,10 @@ class RoutedExperts(FeedForward):
         out.append(TensorSpec(prefix + self.names["router"], (self.E, self.H)))
         if self.router_bias:
             out.append(TensorSpec(prefix + self.names["router_bias"], (self.E,), kind="vector", init="normal"))
+        if self.sigmoid:
+            out.append(TensorSpec(prefix + self.names["correction"], (self.E,), kind="vector", init="normal"))
+        if self.shared is not None:
+            out += self.shared.weight_specs(prefix)
         return out
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
@@ -157,6 +179,10 @@ class RoutedExperts(FeedForward):
         self.w_router = rt.own(tensors[prefix + self.names["router"]])
         if self.router_bias:
             self.b_router = rt.own(tensors[prefix + self.names["router_bias"]].to(torch.float32).reshape(-1))
+        if self.sigmoid:
+            self.correction = rt.own(tensors[prefix + self.names["correction"]].to(torch.float32).reshape(-1))
+        if self.shared is not None:
+            self.shared.load(tensors, prefix, rt)
 
     # from this many tokens a step goes expert by expert through the matrix products (below it, every (token, slot)
     # pair reads its expert's rows itself, which is what a step of few tokens costs anyway)
@@ -169,7 +195,12 @@ class RoutedExperts(FeedForward):
         linear(h, self.w_router, scores, step.ws)
         chosen = step.ws.get("moe_chosen", (T, self.top), torch.int32)
         share = step.ws.get("moe_share", (T, self.top), torch.float32)
-        K.route_topk(scores, self.b_router, chosen, share, self.top, self.out_scale)
+        if self.sigmoid:
+            K.route_sigmoid(scores, self.correction, chosen, share, self.top, self.groups, self.groups_keep, self.out_scale)
+        else:
+            K.route_topk(scores, self.b_router, chosen, share, self.top, self.out_scale)
+        if self.shared is not None:
+            self.shared.forward(h, x, step)          # every token's: added like the experts' outputs
         few = step.is_decode or T < int(os.environ.get("BRAIDINFER_BY_EXPERT_FROM", str(self.BY_EXPERT_FROM)))
         if few and not K.experts_grouped_takes(dt, self.H, self.I):
             # every pair reads its expert's rows itself: the 32-bit path, and widths the grouped kernels do not take

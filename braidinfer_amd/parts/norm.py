@@ -8,7 +8,11 @@ LayerNorm: y = (x - mean) / sqrt(var + eps) * w, var the mean of the squared dev
 and no bias (absent in the reference, whose models norm without centering).
 
 `tensor` is the piece of the weight's name behind the part's prefix ("weight" in the
-checkpoints the reference loads; "" where the prefix is the whole name)."""
+checkpoints the reference loads; "" where the prefix is the whole name).
+
+`rows`: no norm at all, y = x in the compute dtype, for a half of a layer that reads the residual rows themselves
+(a design that norms a half's output only).  It has no weights; a norm that adds behind the half before can leave
+these rows in the same kernel, as it would leave a following norm's."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -113,5 +117,29 @@ class LayerNorm(Norm):
         return nxt is not None
 
 
+class PlainRows(Norm):
+    """The residual rows as they are, in the compute dtype: the "norm" in front of a half that reads the rows themselves."""
+
+    graph_safe = True
+
+    def __init__(self, size: int):
+        self.size = int(size)
+
+    def forward(self, x, out, rows=None):
+        if rows is not None:
+            if out.dtype != x.dtype:
+                raise K.KernelError("rows: chosen rows are gathered in float32 only")
+            K.gather_rows(x, rows, out)
+        elif out.dtype == x.dtype:
+            out.copy_(x)
+        else:
+            K.convert(x, out)
+        return out
+
+    def then_args(self):
+        return None, 0.0, False          # no weight: the kernel behind another norm leaves the rows as they are
+
+
+register_part("norm", "rows", PlainRows, replace=True)
 register_part("norm", "rmsnorm", RMSNorm, replace=True)
 register_part("norm", "layernorm", LayerNorm, replace=True)

@@ -13,6 +13,11 @@ wavelength makes t turns over `original` positions, lo = max(floor(i(fast)), 0),
 rotary_dim - 1) and ramp_p = clamp((p - lo) / max(hi - lo, 0.001), 0, 1), pair p turns with
 inv_freq[p] / factor * ramp_p + inv_freq[p] * (1 - ramp_p) (fast pairs keep their frequency, slow ones are
 slowed by `factor`), and cos and sin are multiplied by 0.1 ln(factor) + 1.  The reference has no such scaling.
+
+`scaling` = {factor, original, low, high} (`scaling_rule` "wavelength") is the other common stretch: a pair whose
+wavelength l = 2 pi / f is shorter than original / high keeps its frequency, one whose wavelength is longer than
+original / low turns with f / factor, and between the two, with s = (original / l - low) / (high - low), with
+(1 - s) f / factor + s f; cos and sin are not scaled.
 """
 from __future__ import annotations
 
@@ -31,7 +36,10 @@ class RotaryEncoding(PositionEncoding):
     graph_safe = True
     gives = "rotary"
 
-    def __init__(self, rotary_dim: int, theta: float, pairing: str = "half", scaling: Optional[Dict[str, float]] = None):
+    def __init__(self, rotary_dim: int, theta: float, pairing: str = "half", scaling: Optional[Dict[str, float]] = None,
+                 scaling_rule: str = "ramp", frequencies_from_float64: bool = False):
+        """`frequencies_from_float64`: the frequencies are worked out in float64 on the host and rounded to float32 once
+        (as with any `scaling`), instead of by float32 powers."""
         if rotary_dim <= 0 or rotary_dim % 2:
             raise ConfigError(f"rotary_dim must be positive and even, got {rotary_dim}")
         if pairing not in ("half", "adjacent"):
@@ -39,7 +47,18 @@ class RotaryEncoding(PositionEncoding):
         self.rotary_dim, self.theta, self.pairing = int(rotary_dim), float(theta), pairing
         self.scaling = None
         self.magnitude = 1.0
-        if scaling is not None:
+        if scaling_rule not in ("ramp", "wavelength"):
+            raise ConfigError(f"rope scaling rule must be 'ramp' or 'wavelength', got {scaling_rule!r}")
+        self.scaling_rule = scaling_rule
+        self.frequencies_from_float64 = bool(frequencies_from_float64)
+        if scaling is not None and scaling_rule == "wavelength":
+            try:
+                self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "low", "high")}
+            except (KeyError, TypeError, ValueError):
+                raise ConfigError(f"rope scaling by wavelength needs the numbers factor, original, low and high, got {scaling!r}") from None
+            if min(self.scaling.values()) <= 0 or self.theta <= 0 or self.scaling["high"] == self.scaling["low"]:
+                raise ConfigError(f"rope scaling by wavelength takes positive numbers with low and high apart, got {scaling!r}")
+        elif scaling is not None:
             try:
                 self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
             except (KeyError, TypeError, ValueError):
@@ -56,6 +75,18 @@ class RotaryEncoding(PositionEncoding):
         sc = self.scaling
         if sc is None:
             return f
+        if self.scaling_rule == "wavelength":
+            out = []
+            for fp in f:
+                wavelength = 2.0 * math.pi / fp
+                if wavelength < sc["original"] / sc["high"]:
+                    out.append(fp)
+                elif wavelength > sc["original"] / sc["low"]:
+                    out.append(fp / sc["factor"])
+                else:
+                    s = (sc["original"] / wavelength - sc["low"]) / (sc["high"] - sc["low"])
+                    out.append((1.0 - s) * fp / sc["factor"] + s * fp)
+            return out
 
         def pair_of(turns):
             return n * math.log(sc["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
@@ -69,7 +100,7 @@ class RotaryEncoding(PositionEncoding):
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        if self.scaling is None:
+        if self.scaling is None and not self.frequencies_from_float64:
             expo = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / float(self.rotary_dim)
             inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32), expo)
         else:
