@@ -150,7 +150,7 @@ def attention_mixer(h, w, p, m, eps, positions):
     """Grouped heads with biased projections, one norm over the whole query (key) projection, partial rotation with
     stretched frequencies, capped scores inside runs of positions, a sink in the softmax, a sigmoid gate a head."""
     T = h.shape[0]
-    H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, e = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
     q = h @ w[p + "q"].T + w[p + "q.b"]
     k = h @ w[p + "k"].T + w[p + "k.b"]
     v = (h @ w[p + "v"].T + w[p + "v.b"]).reshape(T, G, e)
@@ -170,7 +170,7 @@ def attention_mixer(h, w, p, m, eps, positions):
 def retention_mixer(h, w, p, m, eps, positions, state=None):
     """A decayed sum of key-value products per head, read by the rotated query, normed per head, gated."""
     T = h.shape[0]
-    H, d, e = m["heads"], m["dim"], m["vdim"]
+    H, d, e = m["heads"], m["dim"], m.get("vdim", m["dim"])
     q = (h @ w[p + "q"].T).reshape(T, H, d)
     k = (h @ w[p + "k"].T).reshape(T, H, d)
     v = (h @ w[p + "v"].T).reshape(T, H, e)
@@ -188,7 +188,7 @@ def differential_mixer(h, w, p, m, eps, positions):
     """Two softmax maps a head over the same values inside a window that also keeps the first tokens; the second
     map is taken off the first with a learnt factor."""
     T = h.shape[0]
-    H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, e = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
     q = rms_norm((h @ w[p + "q"].T).reshape(T, H, 2, d), w[p + "q.norm"], eps)
     k = rms_norm((h @ w[p + "k"].T).reshape(T, G, 2, d), w[p + "k.norm"], eps)
     v = (h @ w[p + "v"].T).reshape(T, G, e)
@@ -257,18 +257,18 @@ def tensor_shapes(cfg):
             out[p + "norm2"] = (W,)
         p += "mix."
         if layer["type"] == "attention":
-            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            H, G, d, e = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
             for n, rows in (("q", H * d), ("k", G * d), ("v", G * e)):
                 out[p + n] = (rows, W)
                 out[p + n + ".b"] = (rows,)
             out[p + "q.norm"], out[p + "k.norm"] = (H * d,), (G * d,)
             out[p + "sink"], out[p + "g"], out[p + "o"] = (H,), (H, W), (W, H * e)
         elif layer["type"] == "retention":
-            H, d, e = m["heads"], m["dim"], m["vdim"]
+            H, d, e = m["heads"], m["dim"], m.get("vdim", m["dim"])
             out[p + "q"], out[p + "k"], out[p + "v"] = (H * d, W), (H * d, W), (H * e, W)
             out[p + "g"], out[p + "o"] = (H * e, W), (W, H * e)
         else:
-            H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            H, G, d, e = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"])
             out[p + "q"], out[p + "k"], out[p + "v"] = (H * 2 * d, W), (G * 2 * d, W), (G * e, W)
             for n in ("q.norm", "k.norm", "lq1", "lk1", "lq2", "lk2"):
                 out[p + n] = (d,)
@@ -298,9 +298,10 @@ def to_bf16_values(a):
     return u.astype(np.uint32).view(np.float32).astype(np.float64)
 
 
-def random_weights(cfg, seed, router_spread=0.0):
+def random_weights(cfg, seed, router_spread=0.0, gain=1.0):
     """Weights that keep every activation of order one, already rounded to bfloat16.  `router_spread` puts the
-    experts' correction that far apart, so that a bfloat16 run chooses as the float64 run does."""
+    experts' correction that far apart, so that a bfloat16 run chooses as the float64 run does; `gain` sizes the
+    matrices."""
     rng = np.random.default_rng(seed)
     w = {}
     for name, shape in tensor_shapes(cfg).items():
@@ -314,11 +315,12 @@ def random_weights(cfg, seed, router_spread=0.0):
         elif tail in ("lq1", "lk1", "lq2", "lk2"):
             a = 0.3 * rng.standard_normal(shape)
         elif tail == "correction":
-            a = 0.2 * rng.standard_normal(shape) + router_spread * rng.permutation(shape[0])
+            # apart by growing steps, so that no two experts and no two sums of a group's best two come close
+            a = 0.2 * rng.standard_normal(shape) + router_spread * 1.6 ** rng.permutation(shape[0]) * (router_spread > 0)
         elif name == "embed":
             a = rng.standard_normal(shape)
         else:
-            a = rng.standard_normal(shape) * (1.5 / math.sqrt(shape[-1]))
+            a = rng.standard_normal(shape) * (1.5 * gain / math.sqrt(shape[-1]))
         w[name] = to_bf16_values(a)
     return w
 
@@ -343,6 +345,29 @@ def write_safetensors(path, w, dtype="bfloat16"):
         f.write(text)
         for b in blobs:
             f.write(b)
+
+
+def read_model(folder):
+    """(configuration, weights as float64) of a folder with config.json and one model.safetensors."""
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    with open(os.path.join(folder, "model.safetensors"), "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+        data = f.read()
+    w = {}
+    for name, info in header.items():
+        if name == "__metadata__":
+            continue
+        blob = data[info["data_offsets"][0]:info["data_offsets"][1]]
+        if info["dtype"] == "BF16":
+            a = (np.frombuffer(blob, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+        elif info["dtype"] == "F32":
+            a = np.frombuffer(blob, dtype=np.float32)
+        else:
+            raise ValueError(f"{name}: dtype {info['dtype']}")
+        w[name] = a.reshape(info["shape"]).astype(np.float64)
+    return cfg, w
 
 
 def write_model(folder, cfg, w, dtype="bfloat16"):
