@@ -75,7 +75,8 @@ LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_
              "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax", "wkv_scan", "wkv_scan_pieces", "shift_mix", "head_norm_gate", "tanh",
              "latent_prepare", "head_linear", "route_topk", "experts_up", "experts_down", "experts_sort", "experts_gather",
              "experts_combine", "experts_up_grouped", "experts_down_grouped", "experts_gemm", "clamped_glu", "add_bias_rows",
-             "add_position_rows", "pwa_gate", "dr_conv_prepare", "dr_scan", "dr_scan_pieces", "silu_rows"]
+             "add_position_rows", "pwa_gate", "dr_conv_prepare", "dr_scan", "dr_scan_pieces", "silu_rows", "pwa_pair_combine",
+             "route_sigmoid", "dr_rotate_rows"]
 
 
 def kernel_share(torch, eng, entries_of, classes):
@@ -266,7 +267,10 @@ class Shape:
 # equal width and layers; what is set beside a design is a Mistral configuration (a dict) or a preset's name.
 # `--design zivovik`: the Zivovik design beside Sidirax (the library's closest model: attention layers between
 # recurrences over an outer-product state, routed experts) at equal width and number of layer runs.
+# `--design ladadra`: the Ladadra design beside Zivovik (the library's closest model: softmax attention through the
+# same kernels, a decayed sum of key-value products per head, routed experts) at equal width and number of layer runs.
 DESIGN_SIZES = {
+    "ladadra": {"1b": ("ladadra-1b", "zivovik-1b"), "7b": ("ladadra-7b", "zivovik-7b")},
     "zivovik": {"1b": ("zivovik-1b", "sidirax-1b"), "7b": ("zivovik-7b", "sidirax-7b")},
     "sidirax": {"1b": ("sidirax-1b", "kesitar-1b"), "7b": ("sidirax-7b", "kesitar-7b")},
     "kesitar": {
@@ -397,7 +401,7 @@ def design_comparison(args) -> int:
     import torch
     import braidinfer_amd as B
     sizes = DESIGN_SIZES[args.design]
-    beside = {"sidirax": "kesitar", "zivovik": "sidirax"}.get(args.design, "mistral")
+    beside = {"sidirax": "kesitar", "zivovik": "sidirax", "ladadra": "zivovik"}.get(args.design, "mistral")
     line = {"metric": f"{args.design} beside {beside} at equal size: prefill and decode tokens/s, bf16, random weights",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "layers": args.layers or 8,
             "steps": args.steps, "warmup": args.warmup, "sizes": {}}
