@@ -61,7 +61,7 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     T* __restrict__ q_out, T* __restrict__ storage, float* __restrict__ v_first,
     const float* __restrict__ lambda, int vf_role, int nq, int nkv, int dk, int dv, int page,
     int write_cache, int width, int v_col0, float q_coef, int q_every, int maps, const float* __restrict__ row_ss,
-    int nw_stride) {
+    int nw_stride, int pad_q) {
     extern __shared__ float row[];          // [max(dk, dv)]
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int nqs = nq * maps, nks = nkv * maps, kw = maps * dk;     // vectors of dk, and a key row's width
@@ -76,9 +76,10 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     const int p = pos[t];
     T* dst = nullptr;
     if (is_q) {
-        T* qrow = q_out + ((size_t)t * nqs + h) * kw;
-        dst = qrow + map * dk;
-        for (int mm = 0; mm < maps; ++mm)                             // zeros where the other maps' keys lie
+        // `pad_q`: a query row as wide as a key row, with zeros where the other maps' keys lie; else dk wide
+        T* qrow = q_out + ((size_t)t * nqs + h) * (pad_q ? kw : dk);
+        dst = qrow + (pad_q ? map * dk : 0);
+        for (int mm = 0; pad_q && mm < maps; ++mm)
             if (mm != map)
                 for (int i = lane; i < dk; i += 64) qrow[mm * dk + i] = from_f32<T>(0.f);
     } else if (write_cache && slot >= 0) {
@@ -215,8 +216,21 @@ __global__ __launch_bounds__(256) void pwa_row_ss_kernel(const float* __restrict
     const size_t t = blockIdx.x;
     const float* src = qkv + t * width;
     float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < nq_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sq = fmaf(v, v, sq); }
-    for (int i = nq_cols + threadIdx.x; i < nq_cols + nk_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sk = fmaf(v, v, sk); }
+    if (((width | nq_cols | nk_cols) & 3) == 0 && (((uintptr_t)qkv | (uintptr_t)bias) & 15) == 0) {
+        // 16 bytes a load; a thread's elements are added in their order, the threads' sums by a fixed tree
+        const f32x4* s4 = (const f32x4*)src;
+        const f32x4* b4 = (const f32x4*)bias;
+        const int nq4 = nq_cols >> 2, n4 = (nq_cols + nk_cols) >> 2;
+        for (int i = threadIdx.x; i < n4; i += 256) {
+            f32x4 v = s4[i];
+            if (b4) { const f32x4 b = b4[i]; v[0] += b[0]; v[1] += b[1]; v[2] += b[2]; v[3] += b[3]; }
+            const float a = fmaf(v[3], v[3], fmaf(v[2], v[2], fmaf(v[1], v[1], v[0] * v[0])));
+            if (i < nq4) sq += a; else sk += a;
+        }
+    } else {
+        for (int i = threadIdx.x; i < nq_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sq = fmaf(v, v, sq); }
+        for (int i = nq_cols + threadIdx.x; i < nq_cols + nk_cols; i += 256) { const float v = src[i] + (bias ? bias[i] : 0.f); sk = fmaf(v, v, sk); }
+    }
     sq = block_sum(sq, scratch);
     sk = block_sum(sk, scratch);
     if (threadIdx.x == 0) { out[2 * t] = sq; out[2 * t + 1] = sk; }
@@ -229,7 +243,7 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
                               const int* slots, const int* block_table, int table_stride, void* q_out,
                               void* storage, int is_bf16, float* v_first, const float* lambda, int vf_role,
                               int T, int nq, int nkv, int dk, int dv, int page, int write_cache, int width, int v_from_k,
-                              float q_coef, int q_every, int maps, float* row_ss, int nw_stride, hipStream_t s) {
+                              float q_coef, int q_every, int maps, float* row_ss, int nw_stride, int pad_q, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (maps <= 0 || (maps > 1 && v_from_k) || (nw_stride != 0 && nw_stride != dk)) return BR_BAD_ARG;
     const int nqs = nq * maps, nks = nkv * maps, kw = maps * dk;
@@ -252,12 +266,12 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
         pwa_prepare_kernel<bf16><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                        block_table, table_stride, (bf16*)q_out, (bf16*)storage, v_first,
                                                        lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every,
-                                                       maps, row_ss, nw_stride);
+                                                       maps, row_ss, nw_stride, pad_q);
     else
         pwa_prepare_kernel<float><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                         block_table, table_stride, (float*)q_out, (float*)storage,
                                                         v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache, width, v_col0, q_coef, q_every,
-                                                        maps, row_ss, nw_stride);
+                                                        maps, row_ss, nw_stride, pad_q);
     int rc = br_check_launch();
     if (rc != BR_OK || !tiled) return rc;
     dim3 vgrid((T + 63) / 64, nkv, (dv + 63) / 64);
@@ -684,11 +698,13 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
     const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair,
-    int chunk, int keep, float softcap) {
-    const int b = blockIdx.z, kvh = blockIdx.y;
+    int chunk, int keep, float softcap, int maps) {
+    // `maps` > 1: blockIdx.y counts (kv head, map); a query row is dk wide and reads elements map * dk .. of the key
+    // rows, which hold all maps side by side; nq counts the query rows of a token (heads x maps, the map innermost)
+    const int b = blockIdx.z, kvh = blockIdx.y / maps, map = blockIdx.y % maps;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
-    const int G = nq / nkv;
+    const int G = nq / (nkv * maps), kw = maps * dk;
     const int rows_total = n_new * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int row0 = pwa_tile(pair) * 128 + wave * 32;
@@ -697,7 +713,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const int row = row0 + c;
     const bool row_ok = row < rows_total;
     const int rr = row_ok ? row : rows_total - 1;
-    const int tok = rr / G, head = kvh * G + rr % G;
+    const int tok = rr / G, head = (kvh * G + rr % G) * maps + map;
     bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * dv;
     if (slot < 0) {       // padding: no cache behind it
         if (row_ok && g == 0) for (int d = 0; d < dv; ++d) orow[d] = (bf16)0.f;
@@ -726,8 +742,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const float scale2 = scale * PWA_LOG2E;
     const bool capped = softcap > 0.f && scale != 0.f;
     const float cap_in = capped ? 2.0f * PWA_LOG2E * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
-    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
-    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+    const size_t page_elems = (size_t)nkv * PWA_PAGE * (kw + dv);
+    const size_t k_off = (size_t)kvh * PWA_PAGE * kw + (size_t)map * dk, v_off = (size_t)nkv * PWA_PAGE * kw + (size_t)kvh * dv * PWA_PAGE;
 
     if (pool > 0) {
         // blocks wholly before the window: query p sees the pooled rows 0 .. seen(p) - 1
@@ -739,7 +755,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
         for (int kb = 0; kb < seen_max; kb += 32) {
             const int kl = kb % PWA_PAGE;
             const bf16* pg = pooled + (size_t)pt[kb / PWA_PAGE] * page_elems;
-            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, written - kb, 0, seen - 1, dk, dv, c, g,
+            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * kw, kw, pg + v_off + kl, PWA_PAGE, kb, written - kb, 0, seen - 1, dk, dv, c, g,
                                 qf, acc_o, m, lsum, scale2, cap_in, cap_out);
         }
     }
@@ -753,14 +769,14 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
         for (int kb = 0; kb < kept_max; kb += 32) {
             const int kl = kb % PWA_PAGE;
             const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
-            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, 0, kept - 1, dk, dv, c, g,
+            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * kw, kw, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, 0, kept - 1, dk, dv, c, g,
                                 qf, acc_o, m, lsum, scale2, cap_in, cap_out);
         }
     }
     for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
         const int kl = kb % PWA_PAGE;
         const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
-        pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, first_ok, last_ok, dk, dv, c, g,
+        pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * kw, kw, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, first_ok, last_ok, dk, dv, c, g,
                             qf, acc_o, m, lsum, scale2, cap_in, cap_out);
     }
     lsum += __shfl_xor(lsum, 32, 64);
@@ -973,12 +989,13 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
     const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair,
-    int chunk, int keep, float softcap) {
+    int chunk, int keep, float softcap, int maps) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pwa_lds[];
-    const int b = blockIdx.z, kvh = blockIdx.y;
+    // `maps` > 1: as in `pwa_prefill_kernel`; a page's stage holds this map's part of the key rows only
+    const int b = blockIdx.z, kvh = blockIdx.y / maps, map = blockIdx.y % maps;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
-    const int G = nq / nkv;
+    const int G = nq / (nkv * maps), kw = maps * dk;
     const int rows_total = n_new * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wg_row0 = pwa_tile(pair) * 128;
@@ -989,7 +1006,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const int row = row0 + c;
     const bool row_ok = wave_on && row < rows_total;
     const int rr = row_ok ? row : rows_total - 1;
-    const int tok = rr / G, head = kvh * G + rr % G;
+    const int tok = rr / G, head = (kvh * G + rr % G) * maps + map;
     bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * dv;
     if (slot < 0) {       // padding: no cache behind it
         if (row_ok && g == 0) for (int d = 0; d < dv; ++d) orow[d] = (bf16)0.f;
@@ -1019,8 +1036,8 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const float scale2 = scale * PWA_LOG2E;
     const bool capped = softcap > 0.f && scale != 0.f;
     const float cap_in = capped ? 2.0f * PWA_LOG2E * scale / softcap : 0.f, cap_out = capped ? softcap / scale : 0.f;
-    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
-    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+    const size_t page_elems = (size_t)nkv * PWA_PAGE * (kw + dv);
+    const size_t k_off = (size_t)kvh * PWA_PAGE * kw + (size_t)map * dk, v_off = (size_t)nkv * PWA_PAGE * kw + (size_t)kvh * dv * PWA_PAGE;
 
     // what the wave's rows see, and the pages the workgroup walks
     auto seen_of = [&](int p) { const int far = p - size - pool + 1; return (pool > 0 && far >= 0) ? far / pool + 1 : 0; };
@@ -1045,6 +1062,13 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     // a page's keys are PAGE * dk / 8 pieces of 16 bytes, its values dv * 8: each thread brings up to NBK + NBV of each
     const int k_pieces = PWA_PAGE * dk / 8, v_pieces = dv * 8;
     bf16x8 rk[NBK], rv[NBV];
+    // where a thread's pieces of the keys lie in a page: row (piece / pieces a row) of the page's key rows, kw apart
+    int k_src[NBK];
+#pragma unroll
+    for (int i = 0; i < NBK; ++i) {
+        const int piece = threadIdx.x + 256 * i, per = dk / 8;
+        k_src[i] = (piece / per) * kw + (piece % per) * 8;
+    }
     auto page_of = [&](int n) -> const bf16* {
         if (n < far_pages) return pooled + (size_t)pt[n] * page_elems;
         if (n < far_pages + kept_pages) return storage + (size_t)bt[n - far_pages] * page_elems;
@@ -1055,7 +1079,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
 #pragma unroll
         for (int i = 0; i < NBK; ++i) {
             const int piece = threadIdx.x + 256 * i;
-            rk[i] = piece < k_pieces ? *(const bf16x8*)(pg + k_off + (size_t)piece * 8) : pwa_zero8();
+            rk[i] = piece < k_pieces ? *(const bf16x8*)(pg + k_off + k_src[i]) : pwa_zero8();
         }
 #pragma unroll
         for (int i = 0; i < NBV; ++i) {
@@ -1121,7 +1145,7 @@ template <int NBK>
 static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
                                 const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
                                 int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks,
-                                int chunk, int keep, float softcap) {
+                                int chunk, int keep, float softcap, int maps) {
     // steps that fill a workgroup's 128 rows stage the pages in LDS (key widths in steps of 8 and value widths in steps
     // of 8 that the kernel's pieces cover); shorter ones read their operands straight from the cache
     const int cus = br_device_cus();
@@ -1136,8 +1160,8 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
                 if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
                 have = lds; \
             } \
-            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap); \
-        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap); \
+            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap, maps); \
+        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair, chunk, keep, softcap, maps); \
     } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
@@ -1148,22 +1172,24 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
     return br_check_launch();
 }
 
-// Takes bfloat16, widths of keys in steps of 8 and of values in steps of 4, each up to 256.
+// Takes bfloat16, widths of keys in steps of 8 and of values in steps of 4, each up to 256.  `maps` > 1: `nq` counts a
+// token's query rows (heads x maps, the map innermost), each dk wide; the cache's key rows are maps * dk wide, and
+// every (kv head, map) is a workgroup column of its own, so no product is spent on another map's key elements.
 extern "C" int br_pwa_prefill_bf16(const void* q, void* out, const int* cu_seqlens, const int* slots, const int* ctx_lens,
                                    const int* block_table, int table_stride, const void* storage, const int* pooled_table,
                                    int pooled_stride, const void* pooled, int B, int max_new, int nq, int nkv, int dk, int dv,
                                    int size, int pool, float scale, int sink, const float* __restrict__ sinks, int chunk, int keep,
-                                   float softcap, hipStream_t s) {
+                                   float softcap, int maps, hipStream_t s) {
     if (B <= 0 || max_new <= 0) return BR_OK;
-    if (nq <= 0 || nkv <= 0 || nq % nkv || nkv > 65535 || B > 65535 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 ||
+    if (maps <= 0 || nq <= 0 || nkv <= 0 || nq % (nkv * maps) || nkv * maps > 65535 || B > 65535 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 ||
         dv % 4 || size <= 0 || pool < 0 || (pool > 0 && (!pooled_table || !pooled)) || chunk < 0 || keep < 0 || !(softcap >= 0.f))
         return BR_BAD_ARG;
-    const int G = nq / nkv;
-    dim3 grid((unsigned)(((size_t)max_new * G + 127) / 128), nkv, B);
+    const int G = nq / (nkv * maps);
+    dim3 grid((unsigned)(((size_t)max_new * G + 127) / 128), nkv * maps, B);
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
 #define PWA_K(KK) pwa_prefill_launch_v<KK>(nbv, grid, s, (const bf16*)q, (bf16*)out, cu_seqlens, slots, ctx_lens, block_table, table_stride, \
                                            (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, \
-                                           chunk, keep, softcap)
+                                           chunk, keep, softcap, maps)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);

@@ -542,7 +542,7 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
                 block_table: torch.Tensor, q_out: torch.Tensor, unit: torch.Tensor, v_first: Optional[torch.Tensor],
                 mix: Optional[torch.Tensor], v_role: int, nq: int, nkv: int, dk: int, dv: int, page: int,
                 write_cache: bool, values_from_keys: bool = False, q_temp_coef: float = 0.0, q_temp_every: int = 0,
-                maps: int = 1, row_ss: Optional[torch.Tensor] = None) -> None:
+                maps: int = 1, row_ss: Optional[torch.Tensor] = None, pad_queries: bool = True) -> None:
     """Float projection sums [T, nq*dk + nkv*dk + nkv*dv (+ more columns that are not read)] -> queries (normed,
     rotated) in `q_out` and the tokens' keys (normed, rotated) and values in their cache pages.  `v_role` 1 leaves
     the values in `v_first`, 2 mixes them with it by the scalar `mix`.  `values_from_keys`: there are no value
@@ -552,7 +552,8 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
     cache's key rows are maps * dk wide and `q_out` is [T, nq * maps rows of maps * dk], every row one map's query with
     zeros where the other maps' keys lie (the attention kernels then take nq * maps query heads of maps * dk).  `row_ss`
     (float scratch [T, 2]): the norm runs over the token's whole query (key) projection instead of over a head, with
-    weights for the whole projection (`q_norm` [nq * maps * dk], `k_norm` [nkv * maps * dk])."""
+    weights for the whole projection (`q_norm` [nq * maps * dk], `k_norm` [nkv * maps * dk]).  `pad_queries` False: the
+    rows of `q_out` are dk wide, without the zeros (for a kernel that takes `maps` itself)."""
     _dev("pwa_prepare", qkv, bias, q_norm, k_norm, cos, sin, positions, seq_of_token, slots, block_table, q_out, unit,
          v_first, mix, row_ss)
     T = qkv.shape[0]
@@ -572,7 +573,8 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
          "pwa_prepare: a norm over the whole projection takes float scratch [T, 2] and weights for queries and keys")
     _req(positions.numel() >= T and seq_of_token.numel() >= T, "pwa_prepare: positions shorter than tokens")
     _req(block_table.dim() == 2 and block_table.dtype == torch.int32, "pwa_prepare: block table int32 [slots, pages]")
-    _req(q_out.shape == (T, nqs * kw) and q_out.dtype == unit.dtype, "pwa_prepare: q_out [T, nq*maps*maps*dk] of the cache's dtype")
+    _req(q_out.shape == (T, nqs * (kw if pad_queries else dk)) and q_out.dtype == unit.dtype,
+         "pwa_prepare: q_out [T, nq*maps rows of maps*dk (or of dk, without the zeros)] of the cache's dtype")
     _pwa_unit("pwa_prepare", unit, nkv, kw, dv, page)
     if rotary_dim:
         _req(cos is not None and sin is not None and cos.dtype == sin.dtype == torch.float32
@@ -582,12 +584,12 @@ def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optiona
              "pwa_prepare: v_first float32 [T, nkv*dv]")
         _req(v_role != 2 or (mix is not None and mix.dtype == torch.float32 and mix.numel() == 1), "pwa_prepare: mix is one float")
     f = _fn("pooled_attention", "br_pwa_prepare",
-            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 10 + [c_float, c_int, c_int, _P, c_int, _P])
+            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 10 + [c_float, c_int, c_int, _P, c_int, c_int, _P])
     _check(f(_ptr(qkv), _ptr(bias), _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(cos), _ptr(sin), int(rotary_dim),
              _ptr(positions), _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(q_out),
              _ptr(unit), _is_bf16(unit, "pwa_prepare"), _ptr(v_first), _ptr(mix), int(v_role), T, nq, nkv, dk, dv, page,
              int(write_cache), int(qkv.shape[1]), int(bool(values_from_keys)), float(q_temp_coef), int(q_temp_every),
-             int(maps), _ptr(row_ss), dk if whole else 0, _stream()), "pwa_prepare")
+             int(maps), _ptr(row_ss), dk if whole else 0, int(bool(pad_queries)), _stream()), "pwa_prepare")
 
 
 def pwa_pair_combine(a: torch.Tensor, out: torch.Tensor, nq: int, dv: int, factor: float, eps: Optional[float],
@@ -678,9 +680,11 @@ def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tenso
                      block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
                      pooled: Optional[torch.Tensor], B: int, max_new: int, nq: int, nkv: int, dk: int, dv: int, page: int,
                      size: int, pool: int, scale: float, sink: bool, sinks: Optional[torch.Tensor] = None, chunk: int = 0,
-                     keep: int = 0, softcap: float = 0.0) -> None:
+                     keep: int = 0, softcap: float = 0.0, maps: int = 1) -> None:
     """Steps of several tokens per sequence on the matrix cores: the same sums as `pwa_attend`, bfloat16 operands,
-    float scores and softmax, the weights rounded to bfloat16 for the second product."""
+    float scores and softmax, the weights rounded to bfloat16 for the second product.  `maps` > 1: `nq` counts a token's
+    query rows (heads x maps, the map innermost), each `dk` wide (`pwa_prepare` without padding); the cache's key rows hold
+    the maps side by side, and query row (h, m) reads elements m * dk .. (m + 1) * dk of them."""
     _dev("pwa_prefill_bf16", q, out, cu_seqlens, slots, ctx_lens, block_table, unit, pooled_table, pooled)
     T = q.shape[0]
     _req(pwa_prefill_takes(q.dtype, dk, dv, page), "pwa_prefill_bf16: bfloat16, pages of 64, key widths in steps of 8 and value "
@@ -688,16 +692,17 @@ def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tenso
     _req(q.shape == (T, nq * dk) and out.shape == (T, nq * dv) and out.dtype == unit.dtype == torch.bfloat16,
          "pwa_prefill_bf16: q [T, nq*dk], out [T, nq*dv], bfloat16 like the cache")
     _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B and ctx_lens.numel() >= B, "pwa_prefill_bf16: arrays shorter than the batch")
-    _pwa_unit("pwa_prefill_bf16", unit, nkv, dk, dv, page)
+    _req(maps >= 1 and nq % (nkv * maps) == 0 and (maps == 1 or not pool), "pwa_prefill_bf16: query rows a multiple of kv heads x maps; no pooled rows with maps")
+    _pwa_unit("pwa_prefill_bf16", unit, nkv, maps * dk, dv, page)
     if pool:
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_prefill_bf16: pooled unit missing")
         _pwa_unit("pwa_prefill_bf16", pooled, nkv, dk, dv, page)
     f = _fn("pooled_attention", "br_pwa_prefill_bf16",
-            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, c_int, c_int, c_float, _P])
+            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, c_int, c_int, c_float, c_int, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit),
              _ptr(pooled_table), pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, max_new, nq, nkv, dk, dv,
              int(size), int(pool), float(scale), int(sink), _sinks("pwa_prefill_bf16", sinks, nq), int(chunk), int(keep),
-             float(softcap), _stream()), "pwa_prefill_bf16")
+             float(softcap), int(maps), _stream()), "pwa_prefill_bf16")
 
 
 def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, page: int) -> bool:

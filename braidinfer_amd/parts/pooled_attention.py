@@ -246,7 +246,12 @@ class PooledWindowAttention(Mixer):
         qkv = step.ws.get("pwa_qkv", (T, self.gate_col0 + self.n_gate), torch.float32)
         linear(h, self.w_qkv, qkv, step.ws)
         maps, kw = self.maps, self.kw
-        q = step.ws.get("pwa_q", (T, nq * maps * kw), dt)
+        # prompts and portions in bfloat16 go to the matrix cores; with two maps that kernel takes the maps itself (query
+        # rows of key_dim), the others see every map as a query head over key rows that hold all maps (rows of maps * key_dim
+        # with zeros outside the map's own elements)
+        by_matrix_prefill = not step.is_decode and not self.force_simple and K.pwa_prefill_takes(dt, dk, dv, ctx.page_tokens)
+        pad = not (by_matrix_prefill and maps > 1)
+        q = step.ws.get("pwa_q", (T, nq * maps * (kw if pad else dk)), dt)
         row_ss = step.ws.get("pwa_row_ss", (T, 2), torch.float32) if self.norm_over_projection else None
         v_first, role = None, 0
         if self.value_mix is not None:
@@ -266,9 +271,9 @@ class PooledWindowAttention(Mixer):
                       tables.cos if tables else None, tables.sin if tables else None, tables.rotary_dim if tables else 0,
                       step.positions, step.seq_of_token, step.slots, ctx.block_table, q, unit, v_first, self.mix, role,
                       nq, nkv, dk, dv, ctx.page_tokens, ctx.writes_cache, self.values_from_keys,
-                      self.q_temp[0] if self.q_temp else 0.0, self.q_temp[1] if self.q_temp else 0, maps=maps, row_ss=row_ss)
-        # the kernels' view: every map a query head of its own over key rows that hold all maps
-        nq, dk = nq * maps, kw
+                      self.q_temp[0] if self.q_temp else 0.0, self.q_temp[1] if self.q_temp else 0, maps=maps, row_ss=row_ss,
+                      pad_queries=pad)
+        nq, dk = nq * maps, (kw if pad else dk)
         mask = dict(chunk=self.chunk, keep=self.keep_first, softcap=self.softcap)
         pooled = ctx.others.get("pooled")
         if pooled is not None and ctx.writes_cache:
@@ -277,11 +282,10 @@ class PooledWindowAttention(Mixer):
         o = step.ws.get("pwa_out" if maps == 1 else "pwa_out_maps", (T, nq * dv), dt)
         p_table = pooled.block_table if pooled is not None else None
         p_unit = pooled.storage if pooled is not None else None
-        if not step.is_decode and not self.force_simple and K.pwa_prefill_takes(dt, dk, dv, ctx.page_tokens):
-            # prompts and portions in bfloat16: the matrix cores
+        if by_matrix_prefill:
             K.pwa_prefill_bf16(q, o, step.cu_seqlens, step.slots, step.ctx_lens, ctx.block_table, unit, p_table, p_unit,
                                step.n_seqs, step.max_new, nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool,
-                               self.scale, self.sink, self.sinks, **mask)
+                               self.scale, self.sink, self.sinks, maps=1 if pad else maps, **mask)
         elif step.is_decode and not self.force_simple and K.pwa_decode_takes(dt, nq, nkv, dk, dv, ctx.page_tokens):
             # single tokens in bfloat16: the matrix cores, a kv head's keys read once for its query heads
             K.pwa_decode_bf16(q, o, step.slots, step.ctx_lens, ctx.block_table, unit, p_table, p_unit, step.n_seqs,

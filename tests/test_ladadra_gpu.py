@@ -442,6 +442,45 @@ def test_a_sink_that_takes_all_the_weight_and_one_that_takes_none():
         assert np.abs(unbounded - bounded).max() > 0.1
 
 
+@pytest.mark.parametrize("H,G,d,e,T", [(4, 2, 16, 24, 150), (2, 2, 64, 128, 300), (8, 1, 32, 64, 100), (1, 1, 8, 12, 70)])
+def test_two_maps_through_the_matrix_core_kernels(H, G, d, e, T):
+    """Prompts on the matrix cores take the maps as workgroups of their own (query rows of d, reading their map's part
+    of the key rows); single tokens and the float kernel see every map as a query head over whole key rows (zeros outside
+    the map).  Both against the plain attention of every map, whole and behind an earlier portion."""
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(T + d)
+    raw = rng.standard_normal((T, (H + G) * 2 * d + G * e)).astype(np.float32)
+    q, k = bf(raw[:, :H * 2 * d]).reshape(T, H * 2, d), bf(raw[:, H * 2 * d:(H + G) * 2 * d]).reshape(T, G, 2, d)
+    v = bf(raw[:, (H + G) * 2 * d:]).reshape(T, G, e)
+    vis = P.window_mask(T, 70, 9)
+    want = np.zeros((T, H * 2, e))
+    for m in range(2):
+        want[:, m::2] = P.masked_attention(q[:, m::2], k[:, :, m], v, 0.3, vis)
+    n_pages = -(-T // 64)
+    table = shuffled_table(n_pages, 4, 2, T)
+    for padded in (True, False):
+        unit = torch.zeros((n_pages + 3, G * 64 * (2 * d + e)), dtype=torch.bfloat16, device="cuda")
+        got, at = [], 0
+        for n in (T - 40, 38, 1, 1):
+            pos, sot, slots = dev_i(np.arange(at, at + n)), dev_i(np.zeros(n)), dev_i([2])
+            pad = padded or n == 1
+            qo = torch.zeros((n, H * 2 * (2 * d if pad else d)), dtype=torch.bfloat16, device="cuda")
+            K.pwa_prepare(dev_f(raw[at:at + n]), None, None, None, 0.0, None, None, 0, pos, sot, slots, dev_i(table), qo, unit, None, None, 0,
+                          H, G, d, e, 64, True, maps=2, pad_queries=pad)
+            o = torch.full((n, H * 2 * e), 5.0, dtype=torch.bfloat16, device="cuda")
+            if n == 1:
+                K.pwa_decode_bf16(qo, o, slots, dev_i([at + 1]), dev_i(table), unit, None, None, 1, H * 2, G, 2 * d, e, 64, 70, 0, 0.3, False, None, keep=9)
+            elif pad:
+                K.pwa_prefill_bf16(qo, o, dev_i([0, n]), slots, dev_i([at + n]), dev_i(table), unit, None, None, 1, n, H * 2, G, 2 * d, e, 64, 70, 0,
+                                   0.3, False, None, keep=9)
+            else:
+                K.pwa_prefill_bf16(qo, o, dev_i([0, n]), slots, dev_i([at + n]), dev_i(table), unit, None, None, 1, n, H * 2, G, d, e, 64, 70, 0,
+                                   0.3, False, None, keep=9, maps=2)
+            got.append(o.float().cpu().numpy())
+            at += n
+        assert np.abs(np.concatenate(got).reshape(T, H * 2, e) - want).max() < 0.03, f"padded {padded}"
+
+
 def test_two_maps_into_one_head():
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(11)
