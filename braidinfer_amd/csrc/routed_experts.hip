@@ -65,15 +65,24 @@ extern "C" int br_route_topk(const float* scores, const float* bias, int* chosen
 // c = s + correction, the shares on s.  With `groups` > 1 the experts form that many runs of E / groups neighbours; a
 // run's score is the sum of its two largest c (of its one, where a run is one expert), only experts of the `keep`
 // best runs can be chosen (the others count as minus infinity), ties to the lower number everywhere.  The shares are
-// the chosen experts' s over their sum (+ 1e-20), times `out_scale`.  grid (T), one wave a token; LDS: E floats.
+// the chosen experts' s over their sum (+ 1e-20), times `out_scale`.  grid (T), one wave a token.
+// Nothing is found by rounds of wave-wide maxima: every expert counts the experts that go before it (a larger c, or
+// the same c and a lower number) by reading all c from LDS, and is chosen when fewer than `top` do, its count being
+// its place among the chosen; the runs are kept the same way.  LDS: E + groups + 128 words.
+// NPL: experts (and runs) a lane holds, ceil(E / 64) rounded up to 1, 2, 4 or 8.
+template <int NPL>
 __global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restrict__ scores, const float* __restrict__ correction,
                                                            int* __restrict__ chosen, float* __restrict__ share, int E, int top,
                                                            int groups, int keep, float out_scale) {
-    extern __shared__ float cs[];           // the choice scores
+    extern __shared__ float rs_lds[];
+    float* cs = rs_lds;                     // [E] the choice scores
+    float* gsL = cs + E;                    // [groups] the runs' scores, then whether a run is kept
+    float* picked = gsL + groups;           // [64] the chosen experts' s by their place
+    int* who = (int*)(picked + 64);         // [64] the chosen experts by their place
     const int t = blockIdx.x, lane = threadIdx.x;
-    float sg[RX_MAX_PER_LANE], z[RX_MAX_PER_LANE];
+    float sg[NPL], z[NPL];
 #pragma unroll
-    for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+    for (int i = 0; i < NPL; ++i) {
         const int e = lane + 64 * i;
         sg[i] = 0.f;
         z[i] = -INFINITY;
@@ -83,13 +92,14 @@ __global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restri
             cs[e] = z[i];
         }
     }
+    // a place for every slot whatever the scores are (a padding row's may compare with nothing)
+    if (lane < top) { who[lane] = lane; picked[lane] = 0.f; }
+    __syncthreads();
     if (groups > 1) {
-        __syncthreads();
         const int per = E / groups;
-        // lane g scores run g + 64 j; the best `keep` runs are taken one after the other
-        float gs[RX_MAX_PER_LANE];
+        float gs[NPL];
 #pragma unroll
-        for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
+        for (int j = 0; j < NPL; ++j) {
             const int g = lane + 64 * j;
             gs[j] = -INFINITY;
             if (g < groups) {
@@ -99,62 +109,57 @@ __global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restri
                     if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) b2 = v;
                 }
                 gs[j] = per > 1 ? b1 + b2 : b1;
+                gsL[g] = gs[j];
             }
         }
         __syncthreads();
-        for (int e = lane; e < E; e += 64) cs[e] = -INFINITY;      // now: minus infinity unless the expert's run is kept
-        __syncthreads();
-        for (int r = 0; r < keep; ++r) {
-            float best = -INFINITY;
-            int at = 0x7fffffff;
+        int before[NPL];
 #pragma unroll
-            for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
-                const int g = lane + 64 * j;
-                if (g < groups && gs[j] != -INFINITY && (gs[j] > best || (gs[j] == best && g < at)) ) { best = gs[j]; at = g; }
-            }
+        for (int j = 0; j < NPL; ++j) before[j] = 0;
+#pragma unroll 8
+        for (int h = 0; h < groups; ++h) {
+            const float o = gsL[h];
 #pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float ob = __shfl_xor(best, o, WAVE);
-                const int oa = __shfl_xor(at, o, WAVE);
-                if (oa < 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
-            }
-            if (at == 0x7fffffff) break;          // fewer runs with a score than `keep`
-#pragma unroll
-            for (int j = 0; j < RX_MAX_PER_LANE; ++j)
-                if (lane + 64 * j == at) gs[j] = -INFINITY;
-            for (int i = lane; i < per; i += 64) cs[at * per + i] = 0.f;
+            for (int j = 0; j < NPL; ++j) before[j] += (o > gs[j] || (o == gs[j] && h < lane + 64 * j)) ? 1 : 0;
         }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+        for (int j = 0; j < NPL; ++j) {
+            const int g = lane + 64 * j;
+            if (g < groups) gsL[g] = before[j] < keep ? 1.f : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
             const int e = lane + 64 * i;
-            if (e < E && cs[e] != 0.f) z[i] = -INFINITY;
+            if (e < E && gsL[e / per] == 0.f) { z[i] = -INFINITY; cs[e] = -INFINITY; }
+        }
+        __syncthreads();
+    }
+    int place[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) place[i] = 0;
+#pragma unroll 8
+    for (int j = 0; j < E; ++j) {              // eight reads on their way at a time
+        const float o = cs[j];
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) place[i] += (o > z[i] || (o == z[i] && j < lane + 64 * i)) ? 1 : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        const int e = lane + 64 * i;
+        if (e < E && place[i] < top) {
+            who[place[i]] = e;
+            picked[place[i]] = sg[i];
         }
     }
-    float total = 0.f, mine = 0.f;
-    for (int s = 0; s < top; ++s) {
-        float best = -INFINITY, bs = 0.f;
-        int at = 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
-            const int e = lane + 64 * i;
-            if (e < E && (z[i] > best || (z[i] == best && e < at))) { best = z[i]; at = e; bs = sg[i]; }
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ob = __shfl_xor(best, o, WAVE), os = __shfl_xor(bs, o, WAVE);
-            const int oa = __shfl_xor(at, o, WAVE);
-            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; bs = os; }
-        }
-        if (at >= E) { at = s; bs = 0.f; }        // scores that compare with nothing (a padding row's): any expert will do
-        total += bs;
-        if (lane == s) mine = bs;                 // lane s keeps slot s's score
-        if (lane == 0) chosen[(size_t)t * top + s] = at;
-#pragma unroll
-        for (int i = 0; i < RX_MAX_PER_LANE; ++i)
-            if (lane + 64 * i == at) z[i] = -INFINITY;
+    __syncthreads();
+    if (lane < top) {
+        float total = 0.f;
+        for (int s = 0; s < top; ++s) total += picked[s];          // in the order of the places
+        share[(size_t)t * top + lane] = picked[lane] / (total + 1e-20f) * out_scale;
+        chosen[(size_t)t * top + lane] = who[lane];
     }
-    if (lane < top) share[(size_t)t * top + lane] = mine / (total + 1e-20f) * out_scale;
 }
 
 extern "C" int br_route_sigmoid(const float* scores, const float* correction, int* chosen, float* share, int T, int E, int top,
@@ -163,7 +168,11 @@ extern "C" int br_route_sigmoid(const float* scores, const float* correction, in
     if (E <= 0 || E > 64 * RX_MAX_PER_LANE || top <= 0 || top > E || top > 64 || groups <= 0 || E % groups ||
         (groups > 1 && (keep <= 0 || keep > groups)))
         return BR_BAD_ARG;
-    route_sigmoid_kernel<<<T, 64, (size_t)E * sizeof(float), s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    const size_t lds = (size_t)(E + groups + 128) * sizeof(float);
+    if (E <= 64) route_sigmoid_kernel<1><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    else if (E <= 128) route_sigmoid_kernel<2><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    else if (E <= 256) route_sigmoid_kernel<4><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    else route_sigmoid_kernel<8><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
     return br_check_launch();
 }
 
