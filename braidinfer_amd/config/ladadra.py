@@ -290,7 +290,7 @@ def _with(layer, mlp):
 PRESETS: Dict[str, Dict[str, Any]] = {
     "ladadra-tiny": dict(vocab=320, width=96, norm={"eps": 1e-5}, layers=[
         _with(_differential(4, 2, 16, 24, window=40, keep_first=6), _dense(128)),
-        _with(_attention(6, 2, 16, chunk=48, rot_dims=8, scaling={"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}),
+        _with(_attention(6, 2, 16, chunk=48, rot_dims=8, scaling={"factor": 2.0, "low": 1.0, "high": 3.0, "original": 64}),
               _moe(32, 8, 2, groups=4, keep=2, shared=48)),
         _with(_retention(3, 16, 24), _dense(128)),
         _with(_attention(6, 2, 16, chunk=48, rot_dims=8), None)]),

@@ -150,18 +150,18 @@ def test_plain_attention_with_sink_and_bounded_scores():
 def test_plain_rotation_and_stretched_frequencies():
     f = P.rotary_frequencies(8, 100.0)
     assert np.allclose(f, [1.0, 100 ** -0.25, 100 ** -0.5, 100 ** -0.75])
-    sc = {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 40}
+    sc = {"factor": 5.0, "low": 1.0, "high": 4.0, "original": 40}
     g = P.rotary_frequencies(8, 100.0, sc)
     for fi, gi in zip(f, g):
         wl = 2 * math.pi / fi
         if wl < 10:
             assert gi == fi
         elif wl > 40:
-            assert gi == fi / 4
+            assert gi == fi / 5
         else:
             s = (40 / wl - 1.0) / 3.0
-            assert 0 <= s <= 1 and abs(gi - ((1 - s) * fi / 4 + s * fi)) < 1e-15
-    assert g[0] == f[0] and g[-1] == f[-1] / 4 and f[1] / 4 < g[1] < f[1]      # one of each kind
+            assert 0 <= s <= 1 and abs(gi - ((1 - s) * fi / 5 + s * fi)) < 1e-15
+    assert g[0] == f[0] and g[-1] == f[-1] / 5 and f[1] / 5 < g[1] < f[1]      # one of each kind
     # a rotation keeps lengths, passes the elements behind the rotated ones, and scores depend on distances only
     rng = np.random.default_rng(1)
     x, y = rng.standard_normal((1, 1, 10)), rng.standard_normal((1, 1, 10))
