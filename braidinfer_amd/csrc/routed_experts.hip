@@ -69,7 +69,7 @@ extern "C" int br_route_topk(const float* scores, const float* bias, int* chosen
 // Nothing is found by rounds of wave-wide maxima: every expert counts the experts that go before it (a larger c, or
 // the same c and a lower number) by reading all c from LDS, and is chosen when fewer than `top` do, its count being
 // its place among the chosen; the runs are kept the same way.  LDS: E + groups + 128 words.
-// NPL: experts (and runs) a lane holds, ceil(E / 64) rounded up to 1, 2, 4 or 8.
+// NPL: experts (and runs) a lane holds; the launcher takes this kernel up to 64 experts (NPL 1).
 template <int NPL>
 __global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restrict__ scores, const float* __restrict__ correction,
                                                            int* __restrict__ chosen, float* __restrict__ share, int E, int top,
@@ -162,6 +162,100 @@ __global__ __launch_bounds__(64) void route_sigmoid_kernel(const float* __restri
     }
 }
 
+// The same for more than 64 experts, where a lane holds several: the kept runs and then the `top` experts are taken one
+// after the other by rounds of wave-wide maxima (counting places would walk every choice score once per expert a lane
+// holds: 51 us at 256 experts against 9).  LDS: E floats.
+__global__ __launch_bounds__(64) void route_sigmoid_rounds_kernel(const float* __restrict__ scores, const float* __restrict__ correction,
+                                                           int* __restrict__ chosen, float* __restrict__ share, int E, int top,
+                                                           int groups, int keep, float out_scale) {
+    extern __shared__ float cs[];           // the choice scores
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float sg[RX_MAX_PER_LANE], z[RX_MAX_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        sg[i] = 0.f;
+        z[i] = -INFINITY;
+        if (e < E) {
+            sg[i] = 1.0f / (1.0f + expf(-scores[(size_t)t * E + e]));
+            z[i] = sg[i] + (correction ? correction[e] : 0.f);
+            cs[e] = z[i];
+        }
+    }
+    if (groups > 1) {
+        __syncthreads();
+        const int per = E / groups;
+        // lane g scores run g + 64 j; the best `keep` runs are taken one after the other
+        float gs[RX_MAX_PER_LANE];
+#pragma unroll
+        for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
+            const int g = lane + 64 * j;
+            gs[j] = -INFINITY;
+            if (g < groups) {
+                float b1 = -INFINITY, b2 = -INFINITY;
+                for (int i = 0; i < per; ++i) {
+                    const float v = cs[g * per + i];
+                    if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) b2 = v;
+                }
+                gs[j] = per > 1 ? b1 + b2 : b1;
+            }
+        }
+        __syncthreads();
+        for (int e = lane; e < E; e += 64) cs[e] = -INFINITY;      // now: minus infinity unless the expert's run is kept
+        __syncthreads();
+        for (int r = 0; r < keep; ++r) {
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+#pragma unroll
+            for (int j = 0; j < RX_MAX_PER_LANE; ++j) {
+                const int g = lane + 64 * j;
+                if (g < groups && gs[j] != -INFINITY && (gs[j] > best || (gs[j] == best && g < at)) ) { best = gs[j]; at = g; }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, WAVE);
+                const int oa = __shfl_xor(at, o, WAVE);
+                if (oa < 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+            }
+            if (at == 0x7fffffff) break;          // fewer runs with a score than `keep`
+#pragma unroll
+            for (int j = 0; j < RX_MAX_PER_LANE; ++j)
+                if (lane + 64 * j == at) gs[j] = -INFINITY;
+            for (int i = lane; i < per; i += 64) cs[at * per + i] = 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && cs[e] != 0.f) z[i] = -INFINITY;
+        }
+    }
+    float total = 0.f, mine = 0.f;
+    for (int s = 0; s < top; ++s) {
+        float best = -INFINITY, bs = 0.f;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && (z[i] > best || (z[i] == best && e < at))) { best = z[i]; at = e; bs = sg[i]; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, WAVE), os = __shfl_xor(bs, o, WAVE);
+            const int oa = __shfl_xor(at, o, WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; bs = os; }
+        }
+        if (at >= E) { at = s; bs = 0.f; }        // scores that compare with nothing (a padding row's): any expert will do
+        total += bs;
+        if (lane == s) mine = bs;                 // lane s keeps slot s's score
+        if (lane == 0) chosen[(size_t)t * top + s] = at;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i)
+            if (lane + 64 * i == at) z[i] = -INFINITY;
+    }
+    if (lane < top) share[(size_t)t * top + lane] = mine / (total + 1e-20f) * out_scale;
+}
+
 extern "C" int br_route_sigmoid(const float* scores, const float* correction, int* chosen, float* share, int T, int E, int top,
                                 int groups, int keep, float out_scale, hipStream_t s) {
     if (T <= 0) return BR_OK;
@@ -170,9 +264,7 @@ extern "C" int br_route_sigmoid(const float* scores, const float* correction, in
         return BR_BAD_ARG;
     const size_t lds = (size_t)(E + groups + 128) * sizeof(float);
     if (E <= 64) route_sigmoid_kernel<1><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
-    else if (E <= 128) route_sigmoid_kernel<2><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
-    else if (E <= 256) route_sigmoid_kernel<4><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
-    else route_sigmoid_kernel<8><<<T, 64, lds, s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
+    else route_sigmoid_rounds_kernel<<<T, 64, (size_t)E * sizeof(float), s>>>(scores, correction, chosen, share, E, top, groups, keep, out_scale);
     return br_check_launch();
 }
 
